@@ -40,12 +40,16 @@ int nvs_embed_sinusoid(const void* table, int dtype, const int64_t* ids, const i
 int nvs_norm_residual(const void* m, const void* m2, const void* w1, const void* w2, const void* g, int dtype, int64_t n,
                       int width, float eps, float* x, void* xh, void* stream);
 
-/* Input-side norm on the residual stream, with the adds that precede it: x[t, :] += a[t, :] + b[t, :] (a in `dtype`, b 32-bit,
- * either may be NULL), then out[t, :] = group_rms(x[t, :]) * w: every one of `groups` equal consecutive parts of the row is
- * divided by its own sqrt(mean(part^2) + eps). out == NULL: the adds only. With rows != NULL nothing is added and
- * out[r, :] is the norm of x[rows[r], :]. out and w in `dtype`. */
-int nvs_add_group_norm(float* x, const void* a, const float* b, const int32_t* rows, int64_t nrows, const void* w, int dtype,
-                       int width, int groups, float eps, void* out, void* stream);
+/* Input-side norm on the residual stream, with the adds that precede it: x[t, :] += a_mult * a[t, :] + b[t, :] (a in `dtype`,
+ * b 32-bit, either may be NULL), then out[t, :] = group_rms(x[t, :]) * w: every one of `groups` equal consecutive parts of the
+ * row is divided by its own sqrt(mean(part^2) + eps); with center != 0 the part's mean is taken off first and it is divided by
+ * sqrt(mean of squared deviations + eps) (a layer norm without bias). out == NULL: the adds only. With rows != NULL nothing is
+ * added and out[r, :] is the norm of x[rows[r], :]. out and w in `dtype`. */
+int nvs_add_group_norm(float* x, const void* a, float a_mult, const float* b, const int32_t* rows, int64_t nrows, const void* w,
+                       int dtype, int width, int groups, float eps, int center, void* out, void* stream);
+
+/* out[i] = cap * tanh(in[i] * scale / cap), or in[i] * scale with cap <= 0; in `dtype`, out 32-bit. */
+int nvs_scale_softcap(const void* in, int dtype, float scale, float cap, int64_t numel, float* out, void* stream);
 
 /* out[r, :] = g * rms(x[rows[r], :]) in `dtype` (rows == NULL: row r). */
 int nvs_scalar_norm_rows(const float* x, const int32_t* rows, int64_t nrows, int width, const void* g, int dtype, float eps,
@@ -118,10 +122,10 @@ int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, c
  * (rot_dims, rot_freq; 0: not). Token t of portion s sits at position p = ctx0[s] + (t - cu_q[s]) and sees keys j with
  * 0 <= p - j < window (window > 0), or the keys j <= p of its own block, floor(j / chunk) == floor(p / chunk) (chunk > 0; blocks
  * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
- * gate_stride: out *= sigmoid(gate). out [n, H*dv] `dtype`.
+ * gate_stride: out *= sigmoid(gate); with gate_per_head != 0 the gate is [n, H], one entry for all columns of a head. out [n, H*dv] `dtype`.
  * bf16 with d % 8 == 0 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
  * second product as bf16); everything else, and every float32 call, takes the scalar kernel (one wavefront per query). */
-int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int dtype,
+int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_per_head, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H, int G, int d, int dv,
                     float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out, void* stream);
@@ -131,11 +135,12 @@ int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float ep
 int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, int kind, float limit, float alpha, int64_t n, void* out, void* stream);
 
 /* Routing of a mixture of experts, 32-bit. z [n, total] (row stride z_stride): router logits of all `total` entries.
- * s = softmax(z); choice score c = s + correction (NULL: none). Entries form `count` equal groups of neighbours; a group's score
+ * s = softmax(z) (score 0) or sigmoid(z) (score 1); choice score c = s + correction (NULL: none). Entries form `count` equal groups of neighbours; a group's score
  * is its largest c, and only entries of the `keep` best groups can be chosen. The `top` entries with the largest c are chosen:
- * ids [n, top]; wts [n, top] = s[chosen] / (sum of them + 1e-20) * scale. Ties go to the lower index. */
+ * ids [n, top]; wts [n, top] = s[chosen] / (sum of them + 1e-20) * scale, or s[chosen] * scale with renorm == 0. Ties go to
+ * the lower index. */
 int nvs_moe_route(const float* z, int64_t z_stride, const float* correction, int64_t n, int total, int top, int count, int keep, float scale,
-                  int32_t* ids, float* wts, void* stream);
+                  int score, int renorm, int32_t* ids, float* wts, void* stream);
 
 /* Sort the pairs (token, choice) by expert. Pairs whose id >= experts have no rows (pass-through entries). Every expert's rows are
  * padded to whole tiles of tm (16, 64 or 128) rows; cap = nvs_moe_rows(n * top, experts, tm) rows are laid out.
@@ -144,11 +149,12 @@ int64_t nvs_moe_rows(int64_t pairs, int experts, int tm);
 int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts, int tm, int32_t* tile_expert, int32_t* row_token, int32_t* pair_row,
                  void* stream);
 
-/* Grouped product over the planned rows: out[r, :] = W[expert of r] x(r). glu != 0: W [experts, 2 nout, K] (gate rows, then up rows),
- * x(r) = X[row_token[r], :], out = silu(gate) * up; glu == 0: W [experts, nout, K], x(r) = X[r, :]. X, W, out in `dtype`; bf16 with
+/* Grouped product over the planned rows: out[r, :] = W[expert of r] x(r). mode 1: W [experts, 2 nout, K] (gate rows, then up rows),
+ * x(r) = X[row_token[r], :], out = silu(gate) * up; mode 0: W [experts, nout, K], x(r) = X[r, :]; mode 2: W [experts, nout, K],
+ * x(r) = X[row_token[r], :], out = max(W x, 0)^2 (an ungated expert's first product). X, W, out in `dtype`; bf16 with
  * K % 8 == 0 and ldx % 8 == 0 runs on the matrix cores (tm 128: LDS-tiled, for steps with many rows per expert). Padding rows are
  * not written. */
-int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int glu, int nout, int K, const int32_t* tile_expert,
+int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int mode, int nout, int K, const int32_t* tile_expert,
                  const int32_t* row_token, int64_t cap, int tm, void* out, int64_t ldo, void* stream);
 /* tests: 1 routes bf16 calls through the plain kernel as well */
 void nvs_moe_force_plain(int on);
@@ -158,6 +164,22 @@ void nvs_moe_force_plain(int on);
 int nvs_moe_combine(const void* rows, int64_t ldr, const int32_t* pair_row, const float* wts, int top, const void* h, int64_t ldh,
                     const void* shared, const float* shared_gate, int64_t gate_stride, int dtype, int64_t n, int width, void* out,
                     void* stream);
+
+/* Latent attention, around the attention call (nvs_window_attn with one kv head of size kv_rank + rot_dim, values = the latent).
+ * proj [n, stride] (`dtype`) is a fused projection output. Columns q_col .. + q_rank are RMS-normed with q_norm into cq [n, q_rank].
+ * With kv_col >= 0, columns kv_col .. + kv_rank are RMS-normed with kv_norm (the latent c) and the next rot_dim columns are the
+ * shared key part: its leading rot_dims entries turn by pos[t] * rot_freq[i], i < rot_dims / 2, pair (2i, 2i+1) or, with
+ * rot_halves, (i, i + rot_dims / 2); cos and sin are multiplied by rot_mag. Token t goes to cache slot slots[t] (< 0: skipped):
+ * k_cache [slot][kv_rank + rot_dim] = [c | rotated part]; v_cache [page][kv_rank][block_size] = c, transposed inside the page. */
+int nvs_latent_prep(const void* proj, int64_t stride, int dtype, int q_col, int q_rank, const void* q_norm, void* cq, int kv_col,
+                    int kv_rank, int rot_dim, const void* kv_norm, const int64_t* pos, const float* rot_freq, int rot_dims, int rot_halves,
+                    float rot_mag, float eps, int block_size, const int32_t* slots, void* k_cache, void* v_cache, int64_t n, void* stream);
+
+/* out[t, h, 0 .. width) = in[t, h, 0 .. width) with the leading rot_dims entries rotated as above; rows t have strides in_stride /
+ * out_stride, heads in_head / out_head (elements, `dtype`). */
+int nvs_rotate_heads(const void* in, int64_t in_stride, int in_head, void* out, int64_t out_stride, int out_head, int dtype, int H,
+                     int width, const int64_t* pos, const float* rot_freq, int rot_dims, int rot_halves, float rot_mag, int64_t n,
+                     void* stream);
 
 /* Tests and A/B runs: 1 routes bf16 calls through the scalar kernel too; 2 keeps the matrix-core kernel but without sharing
  * K / V tiles through LDS; 0 restores the defaults. */

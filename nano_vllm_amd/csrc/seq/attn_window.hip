@@ -63,7 +63,7 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
 // then every lane accumulates its value columns over the round's keys.
 template <typename T>
 __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, const T* __restrict__ qnorm, float eps,
-                                   const T* __restrict__ gate, int64_t gate_stride, const T* __restrict__ k_cache,
+                                   const T* __restrict__ gate, int64_t gate_stride, int gate_w, const T* __restrict__ k_cache,
                                    const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int64_t bt_stride,
                                    int block_size, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
                                    const int32_t* __restrict__ tseq, int H, int G, int d, int dv, float scale, int window, int chunk,
@@ -149,7 +149,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
     if (c < dv) {
       float o = acc[i] * inv;
       if (gate) {
-        const float gv = ldf(gate + t * gate_stride + (int64_t)h * dv + c);
+        const float gv = ldf(gate + t * gate_stride + (int64_t)h * gate_w + (gate_w == 1 ? 0 : c));
         o *= 1.f / (1.f + expf(-gv));
       }
       stf(out + (t * H + h) * dv + c, o);
@@ -177,7 +177,7 @@ int g_no_lds = 0;          // tests / A-B: 1 keeps every wavefront on its own op
 template <int DK, int DVB, int QT>     // d <= 32 DK, dv <= 16 DVB, QT tiles of 16 queries per wavefront (they share every K / V load)
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
-    int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    int64_t gate_stride, int gate_w, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
     const float* __restrict__ rot_freq, int rot_dims, int bs_shift, bf16_t* __restrict__ out) {
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     if (!valid_q[t]) continue;
     const float inv = 1.f / ls;
     bf16_t* op = out + ((int64_t)row[t] * H + h) * dv;
-    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * dv : nullptr;
+    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * gate_w : nullptr;
 #pragma unroll
     for (int db = 0; db < DVB; ++db)
 #pragma unroll
@@ -363,7 +363,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
         const int c = db * 16 + gq * 4 + r;
         if (c < dv) {
           float o = oacc[t][db][r] * inv;
-          if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
+          if (gp) o *= 1.f / (1.f + expf(-(float)gp[gate_w == 1 ? 0 : c]));
           op[c] = (bf16_t)o;
         }
       }
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
 template <int DK, int DVB, int QT>
 __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ qnorm, float eps, const bf16_t* __restrict__ gate,
-    int64_t gate_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    int64_t gate_stride, int gate_w, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
     const float* __restrict__ rot_freq, int rot_dims, int bs_shift, int hw, bf16_t* __restrict__ out) {
@@ -594,7 +594,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
     if (!valid_q[t]) continue;
     const float inv = 1.f / ls;
     bf16_t* op = out + ((int64_t)row[t] * H + h) * dv;
-    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * dv : nullptr;
+    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * gate_w : nullptr;
 #pragma unroll
     for (int db = 0; db < DVB; ++db)
 #pragma unroll
@@ -602,7 +602,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
         const int c = db * 16 + gq * 4 + r;
         if (c < dv) {
           float o = oacc[t][db][r] * inv;
-          if (gp) o *= 1.f / (1.f + expf(-(float)gp[c]));
+          if (gp) o *= 1.f / (1.f + expf(-(float)gp[gate_w == 1 ? 0 : c]));
           op[c] = (bf16_t)o;
         }
       }
@@ -610,7 +610,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
 }
 
 template <int DK, int DVB, int QT>
-void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
+void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_w,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
                     int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
@@ -623,7 +623,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
       const int bq = (4 / hw) * 16 * QT;
       const int64_t btiles = n / bq + nseq;         // an upper bound: every portion may end with a partial tile
       window_attn_mfma_lds_kernel<DK, DVB, QT><<<dim3((unsigned)btiles, (unsigned)(G * (hpg / hw))), dim3(256), 0, stream>>>(
-          (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
+          (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
           (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq,
           rot_dims, bs_shift, hw, (bf16_t*)out);
       return;
@@ -631,7 +631,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
   }
   const int64_t tiles = n / (16 * QT) + nseq;       // an upper bound: every portion may end with a partial tile
   window_attn_mfma_kernel<DK, DVB, QT><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
-      (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, (const bf16_t*)k_cache,
+      (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims,
       bs_shift, (bf16_t*)out);
 }
@@ -639,15 +639,15 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
 // Long portions (prefill) put two tiles of 16 queries on a wavefront: half the K / V bytes through the vector cache per
 // MFMA; steps of short portions (decoding) keep one tile, which gives more wavefronts.
 template <int DK, int DVB>
-void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
+void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_w,
                  const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                  const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
                  int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
   if (n >= 32ll * nseq)
-    launch_mfma_qt<DK, DVB, 2>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
+    launch_mfma_qt<DK, DVB, 2>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
                                ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
   else
-    launch_mfma_qt<DK, DVB, 1>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
+    launch_mfma_qt<DK, DVB, 1>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
                                ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
 }
 }  // namespace
@@ -675,7 +675,7 @@ extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, i
 }
 
 extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
-                               int dtype, const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride,
+                               int gate_per_head, int dtype, const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride,
                                int block_size, const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H,
                                int G, int d, int dv, float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out,
                                void* stream) {
@@ -686,11 +686,12 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
   NVS_REQUIRE(H > 0 && H <= 65535 && G > 0 && H % G == 0 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && block_size > 0 && n >= 0,
               "nvs_window_attn: H %d G %d d %d dv %d block %d", H, G, d, dv, block_size);
   if (n == 0 || nseq == 0) return NVS_OK;
+  const int gate_w = gate_per_head ? 1 : dv;         // gate entries per head: one for the whole head, or one per value column
   if (dtype == NVS_BF16 && d % 8 == 0 && block_size % 8 == 0 && !g_force_scalar) {
     const int dk = d <= 64 ? 2 : (d <= 128 ? 4 : 8), dvb = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
 #define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
   if (dk == DK && dvb == DVB)                                                                                                   \
-    launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
+    launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
                          ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, (hipStream_t)stream);
     NVS_MFMA_CASE(2, 4) NVS_MFMA_CASE(2, 8) NVS_MFMA_CASE(2, 16) NVS_MFMA_CASE(4, 4) NVS_MFMA_CASE(4, 8) NVS_MFMA_CASE(4, 16)
     NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 16)
@@ -698,7 +699,7 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
     return nvs_check_launch("nvs_window_attn (matrix cores)");
   }
   NVS_DISPATCH(dtype, window_attn_kernel<T><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
-                          (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, (const T*)k_cache, (const T*)v_cache,
+                          (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache, (const T*)v_cache,
                           block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, (T*)out));
   return nvs_check_launch("nvs_window_attn");
 }

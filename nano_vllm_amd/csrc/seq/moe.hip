@@ -23,6 +23,13 @@ __device__ __forceinline__ float glu_value(float g, float u, int kind, float lim
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);              // clamped: g sigmoid(alpha g) (u + 1)
 }
 
+// ungated products: mode 2 squares the positive part (the input rows are then gathered by token, as for a gated product)
+__device__ __forceinline__ float plain_value(float v, int mode) {
+  if (mode != 2) return v;
+  v = fmaxf(v, 0.f);
+  return v * v;
+}
+
 template <typename T>
 __global__ void glu_act_kernel(const T* __restrict__ gu, int64_t stride, int ff, int kind, float limit, float alpha, int64_t n,
                                T* __restrict__ out) {
@@ -38,7 +45,8 @@ __global__ void glu_act_kernel(const T* __restrict__ gu, int64_t stride, int ff,
 constexpr int ROUTE_PER_LANE = MAX_EXPERTS / 64;
 
 __global__ void moe_route_kernel(const float* __restrict__ z, int64_t z_stride, const float* __restrict__ correction, int total,
-                                 int top, int count, int keep, float scale, int32_t* __restrict__ ids, float* __restrict__ wts) {
+                                 int top, int count, int keep, float scale, int score, int renorm, int32_t* __restrict__ ids,
+                                 float* __restrict__ wts) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
   const int per = total / count;
@@ -55,10 +63,11 @@ __global__ void moe_route_kernel(const float* __restrict__ z, int64_t z_stride, 
 #pragma unroll
   for (int i = 0; i < ROUTE_PER_LANE; ++i) {
     const int e = lane + 64 * i;
-    s[i] = e < total ? expf(s[i] - mx) : 0.f;
+    if (score == 1) s[i] = e < total ? 1.f / (1.f + expf(-s[i])) : 0.f;      // sigmoid: every entry on its own
+    else s[i] = e < total ? expf(s[i] - mx) : 0.f;
     sum += s[i];
   }
-  sum = wave_sum(sum);
+  sum = score == 1 ? 1.f : wave_sum(sum);
 #pragma unroll
   for (int i = 0; i < ROUTE_PER_LANE; ++i) {
     const int e = lane + 64 * i;
@@ -121,7 +130,7 @@ __global__ void moe_route_kernel(const float* __restrict__ z, int64_t z_stride, 
     sv = wave_sum(sv);                              // one lane holds it
     if (lane == k) chosen_s = sv, chosen_e = cand;
   }
-  const float denom = wave_sum(lane < top ? chosen_s : 0.f) + 1e-20f;
+  const float denom = renorm ? wave_sum(lane < top ? chosen_s : 0.f) + 1e-20f : 1.f;
   if (lane < top) {
     ids[t * top + lane] = chosen_e;
     wts[t * top + lane] = chosen_s / denom * scale;
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
 template <typename T, bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ X, int64_t ldx, const T* __restrict__ W, int nout, int K,
                                                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ row_token,
-                                                       int tm, T* __restrict__ out, int64_t ldo) {
+                                                       int tm, T* __restrict__ out, int64_t ldo, int mode) {
   const int tiles_per = tm / 16;
   const int tile = blockIdx.x / tiles_per;
   const int e = tile_expert[tile];
@@ -195,7 +204,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ X, 
   const int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
   const int tok = row_token[r];
   if (tok < 0) return;
-  const int64_t src = GLU ? tok : r;
+  const int64_t src = (GLU || mode == 2) ? tok : r;
   const T* xr = X + src * ldx;
   const T* We = W + (int64_t)e * (GLU ? 2 : 1) * nout * K;
   const int f0 = blockIdx.y * 64 + (threadIdx.x >> 4) * 4;
@@ -212,7 +221,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ X, 
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    if (f0 + i < nout) stf(out + r * ldo + f0 + i, GLU ? glu_value(ag[i], au[i], 0, 0.f, 0.f) : ag[i]);
+    if (f0 + i < nout) stf(out + r * ldo + f0 + i, GLU ? glu_value(ag[i], au[i], 0, 0.f, 0.f) : plain_value(ag[i], mode));
 }
 
 // matrix-core form (bf16, K % 8 == 0, 16-byte aligned rows). Computed transposed, C^T[features x rows] = W X^T with
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ X, 
 template <int MT, bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ X, int64_t ldx, const bf16_t* __restrict__ W, int nout,
                                                             int K, const int32_t* __restrict__ tile_expert,
-                                                            const int32_t* __restrict__ row_token, bf16_t* __restrict__ out, int64_t ldo) {
+                                                            const int32_t* __restrict__ row_token, bf16_t* __restrict__ out, int64_t ldo, int mode) {
   constexpr int FT = 2, NG = GLU ? 2 : 1;
   const int e = tile_expert[blockIdx.x];
   if (e < 0) return;
@@ -235,7 +244,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
     const int64_t r = row0 + mt * 16 + li;
     const int tok = row_token[r];
     xok[mt] = tok >= 0;
-    xp[mt] = X + (xok[mt] ? (GLU ? (int64_t)tok : r) : 0) * ldx + lk;
+    xp[mt] = X + (xok[mt] ? ((GLU || mode == 2) ? (int64_t)tok : r) : 0) * ldx + lk;
   }
   const bf16_t* We = W + (int64_t)e * NG * nout * K;
   const int fbase = blockIdx.y * (64 * FT) + wave * (16 * FT);
@@ -281,7 +290,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (f + i < nout) {
-          const float v = GLU ? glu_value(acc[0][ft][mt][i], acc[NG - 1][ft][mt][i], 0, 0.f, 0.f) : acc[0][ft][mt][i];
+          const float v = GLU ? glu_value(acc[0][ft][mt][i], acc[NG - 1][ft][mt][i], 0, 0.f, 0.f) : plain_value(acc[0][ft][mt][i], mode);
           out[r * ldo + f + i] = (bf16_t)v;
         }
       }
@@ -300,7 +309,7 @@ template <bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __restrict__ X, int64_t ldx, const bf16_t* __restrict__ W, int nout,
                                                              int K, const int32_t* __restrict__ tile_expert,
                                                              const int32_t* __restrict__ row_token, int tiles_m, int tiles_n,
-                                                             bf16_t* __restrict__ out, int64_t ldo) {
+                                                             bf16_t* __restrict__ out, int64_t ldo, int mode) {
   constexpr int BM = 128, BW = 128, BK = 64, LDK = BK + 8, NG = GLU ? 2 : 1, FB = 4 / NG, BN = BW / NG;   // BN features per tile
   __shared__ __attribute__((aligned(16))) bf16_t Xs[BM][LDK];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[BW][LDK];      // GLU: rows [0, 64) gate, [64, 128) up of the tile's features
@@ -322,7 +331,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __res
   for (int i = 0; i < 4; ++i) {
     const int r = sr + 32 * i;
     const int tok = row_token[row0 + r];
-    xsrc[i] = tok >= 0 ? X + (GLU ? (int64_t)tok : row0 + r) * ldx + sk : nullptr;
+    xsrc[i] = tok >= 0 ? X + ((GLU || mode == 2) ? (int64_t)tok : row0 + r) * ldx + sk : nullptr;
     const int g = r / BN, f = ft * BN + r % BN;
     wsrc[i] = f < nout ? We + ((int64_t)g * nout + f) * K + sk : nullptr;
   }
@@ -379,7 +388,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16_t* __res
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (f + i < nout) {
-          const float v = GLU ? glu_value(acc[fb][rb][i], acc[GLU ? fb + FB : fb][rb][i], 0, 0.f, 0.f) : acc[fb][rb][i];
+          const float v = GLU ? glu_value(acc[fb][rb][i], acc[GLU ? fb + FB : fb][rb][i], 0, 0.f, 0.f) : plain_value(acc[fb][rb][i], mode);
           out[r * ldo + f + i] = (bf16_t)v;
         }
       }
@@ -426,13 +435,13 @@ extern "C" int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, in
 }
 
 extern "C" int nvs_moe_route(const float* z, int64_t z_stride, const float* correction, int64_t n, int total, int top, int count, int keep,
-                             float scale, int32_t* ids, float* wts, void* stream) {
-  NVS_REQUIRE(z && ids && wts && n >= 0, "nvs_moe_route: null argument");
+                             float scale, int score, int renorm, int32_t* ids, float* wts, void* stream) {
+  NVS_REQUIRE(z && ids && wts && n >= 0 && (score == 0 || score == 1), "nvs_moe_route: bad argument");
   NVS_REQUIRE(total > 0 && total <= MAX_EXPERTS && z_stride >= total && top > 0 && top <= 64 && count > 0 && count <= 64 && total % count == 0 &&
                   keep > 0 && keep <= count && (int64_t)keep * (total / count) >= top,
               "nvs_moe_route: %d entries, %d choices, %d of %d groups", total, top, keep, count);
   if (n == 0) return NVS_OK;
-  moe_route_kernel<<<dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream>>>(z, z_stride, correction, total, top, count, keep, scale, ids, wts);
+  moe_route_kernel<<<dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream>>>(z, z_stride, correction, total, top, count, keep, scale, score, renorm, ids, wts);
   return nvs_check_launch("nvs_moe_route");
 }
 
@@ -449,9 +458,10 @@ extern "C" int nvs_moe_plan(const int32_t* ids, int64_t n, int top, int experts,
   return nvs_check_launch("nvs_moe_plan");
 }
 
-extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int glu, int nout, int K, const int32_t* tile_expert,
+extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int mode, int nout, int K, const int32_t* tile_expert,
                             const int32_t* row_token, int64_t cap, int tm, void* out, int64_t ldo, void* stream) {
-  NVS_REQUIRE(X && W && tile_expert && row_token && out, "nvs_moe_gemm: null argument");
+  NVS_REQUIRE(X && W && tile_expert && row_token && out && mode >= 0 && mode <= 2, "nvs_moe_gemm: bad argument");
+  const int glu = mode == 1;
   NVS_REQUIRE(nout > 0 && K > 0 && ldx >= K && ldo >= nout && (tm == 16 || tm == 64 || tm == 128) && cap >= 0 && cap % tm == 0,
               "nvs_moe_gemm: %d x %d, %lld rows in tiles of %d", nout, K, (long long)cap, tm);
   if (cap == 0) return NVS_OK;
@@ -464,17 +474,17 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
     NVS_REQUIRE(blocks < (1ll << 31), "nvs_moe_gemm: step too large");
     if (glu)
       moe_gemm_tiled_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert,
-                                                                                row_token, tiles_m, tiles_n, (bf16_t*)out, ldo);
+                                                                                row_token, tiles_m, tiles_n, (bf16_t*)out, ldo, mode);
     else
       moe_gemm_tiled_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert,
-                                                                                 row_token, tiles_m, tiles_n, (bf16_t*)out, ldo);
+                                                                                 row_token, tiles_m, tiles_n, (bf16_t*)out, ldo, mode);
     return nvs_check_launch("nvs_moe_gemm (matrix cores, LDS tiles)");
   }
   if (matrix_cores) {
     const dim3 grid((unsigned)(cap / tm), (unsigned)((nout + 127) / 128));
 #define NVS_MOE_CASE(MT, GLU)                                                                                                        \
   moe_gemm_mfma_kernel<MT, GLU><<<grid, dim3(256), 0, st>>>((const bf16_t*)X, ldx, (const bf16_t*)W, nout, K, tile_expert, row_token,  \
-                                                            (bf16_t*)out, ldo)
+                                                            (bf16_t*)out, ldo, mode)
     if (tm == 64) {
       if (glu) NVS_MOE_CASE(4, true); else NVS_MOE_CASE(4, false);
     } else {
@@ -486,10 +496,10 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
   const dim3 grid((unsigned)(cap / 16), (unsigned)((nout + 63) / 64));
   if (glu) {
     NVS_DISPATCH(dtype, moe_gemm_kernel<T, true><<<grid, dim3(256), 0, st>>>((const T*)X, ldx, (const T*)W, nout, K, tile_expert, row_token, tm,
-                                                                            (T*)out, ldo));
+                                                                            (T*)out, ldo, mode));
   } else {
     NVS_DISPATCH(dtype, moe_gemm_kernel<T, false><<<grid, dim3(256), 0, st>>>((const T*)X, ldx, (const T*)W, nout, K, tile_expert, row_token,
-                                                                             tm, (T*)out, ldo));
+                                                                             tm, (T*)out, ldo, mode));
   }
   return nvs_check_launch("nvs_moe_gemm");
 }

@@ -20,7 +20,7 @@ int nvs_check_launch(const char* what) {
   }
   return NVS_OK;
 }
-extern "C" int nvs_abi_version(void) { return 3; }   // 3: block masks and rotation in attention, pre-norm kernels, decay scan, routed experts
+extern "C" int nvs_abi_version(void) { return 4; }   // 4: centered norms and scaled adds, latent attention, sigmoid routers, logit cap
 extern "C" const char* nvs_last_error(void) { return g_err; }
 
 namespace {
@@ -112,16 +112,17 @@ __global__ void xielu_kernel(const T* __restrict__ in, const T* __restrict__ pq,
   }
 }
 
-// Input-side ("pre") norm on the 32-bit residual: x[t] += a[t] + b[t] first (either may be absent), then every one of
-// `groups` equal parts of the row is divided by its own root mean square and the row is multiplied by w. One workgroup per
+// Input-side ("pre") norm on the 32-bit residual: x[t] += a_mult * a[t] + b[t] first (either may be absent), then every one of
+// `groups` equal parts of the row is divided by its own root mean square — or, with `center`, its mean is taken off first and
+// it is divided by its standard deviation (a layer norm without bias) — and the row is multiplied by w. One workgroup per
 // row; a group is served by one wavefront (several groups per wavefront, in turn, when there are more groups than wavefronts)
 // or by `blockDim / 64 / groups` wavefronts together when there are fewer. With `rows` the kernel only reads:
 // out[r] = norm(x[rows[r]]).
 template <typename T>
-__global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict__ a, const float* __restrict__ b,
+__global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict__ a, float a_mult, const float* __restrict__ b,
                                       const int32_t* __restrict__ rows, const T* __restrict__ w, int width, int groups, float eps,
-                                      T* __restrict__ out) {
-  __shared__ float red[16];
+                                      int center, T* __restrict__ out) {
+  __shared__ float red[2][16];
   const int64_t r = blockIdx.x;
   const int64_t t = rows ? (int64_t)rows[r] : r;
   const int gsz = width / groups, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -130,24 +131,50 @@ __global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict
   const int first = wave / wpg, step = nw / wpg, idx = (wave % wpg) * 64 + lane, stride = wpg * 64;
   for (int g = first; g < groups; g += step) {
     const int c0 = g * gsz;
-    float ss = 0.f;
+    float ss = 0.f, sm = 0.f;
     for (int c = idx; c < gsz; c += stride) {
       float v = xr[c0 + c];
-      if (a) v += ldf(a + t * width + c0 + c);
+      if (a) v += a_mult * ldf(a + t * width + c0 + c);
       if (b) v += b[t * width + c0 + c];
       if (a || b) xr[c0 + c] = v;
       ss += v * v;
+      sm += v;
     }
     if (!out) continue;                             // (uniform over the workgroup)
+    float mean = 0.f;
+    if (center) {                                   // the mean first, then the squared deviations (this thread wrote xr[c0 + c])
+      sm = wave_sum(sm);
+      if (wpg > 1) {
+        if (lane == 0) red[1][wave] = sm;
+        __syncthreads();
+        sm = 0.f;
+        for (int i = 0; i < wpg; ++i) sm += red[1][first * wpg + i];
+      }
+      mean = sm / (float)gsz;
+      ss = 0.f;
+      for (int c = idx; c < gsz; c += stride) {
+        const float dv = xr[c0 + c] - mean;
+        ss += dv * dv;
+      }
+    }
     ss = wave_sum(ss);
     if (wpg > 1) {                                  // (then every wavefront runs this loop exactly once)
-      if (lane == 0) red[wave] = ss;
+      if (lane == 0) red[0][wave] = ss;
       __syncthreads();
       ss = 0.f;
-      for (int i = 0; i < wpg; ++i) ss += red[first * wpg + i];
+      for (int i = 0; i < wpg; ++i) ss += red[0][first * wpg + i];
     }
     const float k = 1.f / sqrtf(ss / (float)gsz + eps);
-    for (int c = idx; c < gsz; c += stride) stf(out + r * width + c0 + c, xr[c0 + c] * k * ldf(w + c0 + c));   // (this thread wrote xr[c0 + c])
+    for (int c = idx; c < gsz; c += stride) stf(out + r * width + c0 + c, (xr[c0 + c] - mean) * k * ldf(w + c0 + c));
+  }
+}
+
+// logits <- cap * tanh(logits * scale / cap) (cap <= 0: logits * scale), 32-bit out
+template <typename T>
+__global__ void scale_softcap_kernel(const T* __restrict__ in, float scale, float cap, int64_t numel, float* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel; i += (int64_t)gridDim.x * blockDim.x) {
+    const float z = ldf(in + i) * scale;
+    out[i] = cap > 0.f ? cap * tanhf(z / cap) : z;
   }
 }
 
@@ -192,8 +219,8 @@ extern "C" int nvs_xielu(const void* in, const void* pq, float beta, int dtype, 
   return nvs_check_launch("nvs_xielu");
 }
 
-extern "C" int nvs_add_group_norm(float* x, const void* a, const float* b, const int32_t* rows, int64_t nrows, const void* w, int dtype,
-                                  int width, int groups, float eps, void* out, void* stream) {
+extern "C" int nvs_add_group_norm(float* x, const void* a, float a_mult, const float* b, const int32_t* rows, int64_t nrows, const void* w,
+                                  int dtype, int width, int groups, float eps, int center, void* out, void* stream) {
   NVS_REQUIRE(x && nrows >= 0 && width > 0 && groups > 0 && width % groups == 0 && (!out || w), "nvs_add_group_norm: width %d groups %d",
               width, groups);
   NVS_REQUIRE(!rows || (!a && !b), "nvs_add_group_norm: selected rows are only read");
@@ -202,6 +229,15 @@ extern "C" int nvs_add_group_norm(float* x, const void* a, const float* b, const
   int threads = 64 * (groups < 4 ? groups : 4);
   if (groups < 4 && 4 % groups == 0 && width / groups >= 512) threads = 256;
   NVS_DISPATCH(dtype, add_group_norm_kernel<T><<<dim3((unsigned)nrows), dim3(threads), 0, (hipStream_t)stream>>>(
-                          x, (const T*)a, b, rows, (const T*)w, width, groups, eps, (T*)out));
+                          x, (const T*)a, a_mult, b, rows, (const T*)w, width, groups, eps, center, (T*)out));
   return nvs_check_launch("nvs_add_group_norm");
+}
+
+extern "C" int nvs_scale_softcap(const void* in, int dtype, float scale, float cap, int64_t numel, float* out, void* stream) {
+  NVS_REQUIRE(in && out && numel >= 0, "nvs_scale_softcap: bad argument");
+  if (numel == 0) return NVS_OK;
+  const int64_t blocks = (numel + 255) / 256;
+  NVS_DISPATCH(dtype, scale_softcap_kernel<T><<<dim3((unsigned)(blocks > 65536 ? 65536 : blocks)), dim3(256), 0, (hipStream_t)stream>>>(
+                          (const T*)in, scale, cap, numel, out));
+  return nvs_check_launch("nvs_scale_softcap");
 }

@@ -890,7 +890,8 @@ class ModelRunner:
 
     def _allocate_stateful_caches(self):
         cfg = self.config
-        kv_layers = [m for m in self.model.modules() if hasattr(m, "kv_shapes")]
+        # (a layer whose kv_shapes() is None reads the pages of another layer and owns none)
+        kv_layers = [m for m in self.model.modules() if hasattr(m, "kv_shapes") and m.kv_shapes() is not None]
         st_layers = [m for m in self.model.modules() if hasattr(m, "state_shapes")]
         esize = torch.finfo(self.dtype).bits // 8
         per_token = sum(int(np.prod(k)) + int(np.prod(v)) for k, v in (m.kv_shapes() for m in kv_layers)) * esize

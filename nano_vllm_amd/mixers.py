@@ -4,6 +4,10 @@
                       query / value head size, optional per-head q/k RMS norm, optional rotation of the leading dimensions
                       in interleaved pairs, optional sigmoid output gate
   AttentionMixer      fused biased q | k | v projection -> WindowAttention -> out projection
+  LatentAttentionMixer  attention whose keys and values are up-projections of a cached low-rank latent plus one rotated key part
+                      shared by the heads; runs in the latent space on WindowAttention's kernels (one kv head), with a query
+                      latent, either rotary pairing, optional frequency scaling, window or causal mask, optional per-head
+                      sigmoid gate, and optionally the cache of an earlier layer instead of its own
   LightningMixer      linear attention as a decaying outer-product recurrence (per-head constant decay), SiLU on q / k / v,
                       RMS norm over the heads together, sigmoid gate
   SSDMixer            state-space-duality (Mamba-2 style) mixer: stateful causal convolution + SiLU, the recurrence in
@@ -12,8 +16,9 @@
   ParallelMixer       two mixers on the same input; the caller averages their RMS-normed outputs
   XIELUFeedForward    up -> xIELU -> down
   ClampedGLU          [gate | up] -> min(g, limit) sigmoid(alpha g) (clamp(u) + 1) -> down
-  RoutedExperts       mixture of gated experts: softmax router with a choice-only correction, choice limited to the best
-                      groups of experts, pass-through experts, optional shared expert with a sigmoid gate per token
+  RoutedExperts       mixture of experts (gated SiLU units, or ungated squared-ReLU units): softmax or sigmoid router with a
+                      choice-only correction, choice limited to the best groups of experts, weights renormalised or not,
+                      pass-through experts, optional shared expert with a sigmoid gate per token
 
 Every constant a design may change is a constructor argument. Matrix products are the vendor library's (F.linear /
 baddbmm); everything else is a kernel of libnvl_seq.so (ops_seq). Layers read the step's packed-portion description from
@@ -107,6 +112,100 @@ class AttentionMixer(nn.Module):
         proj = F.linear(xh, self.in_w, self.in_b)
         q, k, v = self.cols
         return F.linear(self.attn(proj[:, :q], proj[:, q:q + k], proj[:, q + k:], None, positions), self.o_w)
+
+
+def rotary_frequencies(dims: int, base: float, scaling: dict | None = None) -> tuple[list[float], float]:
+    """Frequencies of the dims / 2 rotated pairs, base^(-2i/dims), in double precision, and the factor on cos and sin (1).
+    With `scaling` = {factor, original, fast, slow} (YaRN): pairs that turn fewer than `slow` times over `original` positions have
+    their frequency divided by `factor`, pairs that turn more than `fast` times keep it, the pairs between the two marks
+    (rounded outwards to whole pairs) blend linearly, and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    import math
+    freq = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return freq, 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+
+    def mark(turns: float) -> float:
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+    lo, hi = max(math.floor(mark(float(scaling["fast"]))), 0), min(math.ceil(mark(float(scaling["slow"]))), dims - 1)
+    span = max(hi - lo, 0.001)
+    ramps = [min(max((i - lo) / span, 0.0), 1.0) for i in range(dims // 2)]
+    return [f / factor * r + f * (1.0 - r) for f, r in zip(freq, ramps)], 0.1 * math.log(factor) + 1.0
+
+
+class LatentAttentionMixer(nn.Module):
+    """Attention over a cached latent. Per token the layer keeps c = rms(W_dkv h)[:kv_rank] * w (the latent) and ONE rotated key
+    part of rot_dim entries (the last rows of W_dkv, not normed); head a's key is [W_uk,a c | rotated part], its value W_uv,a c.
+    Queries come from a latent too: q = W_uq (rms(W_dq h) * w), per head [dim unrotated | rot_dim rotated].
+
+    The attention runs in the latent space, which is the same sum reordered: the query of head a becomes
+    [W_uk,a^T q_a | rotated q part] (kv_rank + rot_dim entries), the cached row [c | rotated key part] is the key of ALL heads and
+    c itself the value; W_uv,a is applied to the attention output. That is WindowAttention's paged kernel with one kv head.
+
+    ONE fused in-projection [dq | dkv | gate]; two batched products per head (W_uk^T on the query, W_uv on the output).
+    window > 0: the last `window` positions, else causal. rot_dims (<= rot_dim) leading entries of the rotated parts turn; the pair
+    of i is (2i, 2i+1), or (i, i + rot_dims / 2) with rot_halves. gated: head a's output times sigmoid(W_g h)_a.
+    source: an earlier layer's mixer whose cache this layer reads instead of keeping one (it then has no W_dkv)."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int, scale: float, eps: float,
+                 block_size: int, window: int = 0, rot_dims: int | None = None, rot_base: float = 10000.0, rot_halves: bool = False,
+                 rot_scaling: dict | None = None, gated: bool = False, source: "LatentAttentionMixer | None" = None):
+        super().__init__()
+        rot_dims = rot_dim if rot_dims is None else int(rot_dims)
+        assert rot_dims % 2 == 0 and 0 <= rot_dims <= rot_dim
+        assert kv_rank + rot_dim <= 256, f"latent row of {kv_rank} + {rot_dim} entries: the attention kernels take up to 256"
+        self.H, self.d, self.dr, self.dv, self.qr, self.r = heads, dim, rot_dim, vdim, q_rank, kv_rank
+        self.scale, self.eps, self.window, self.gated, self.block_size = float(scale), eps, int(window), bool(gated), block_size
+        self._source = (source,) if source is not None else ()          # (a tuple: not a submodule of this layer)
+        if source is not None:
+            assert source.r == kv_rank and source.dr == rot_dim and not source._source, "the borrowed cache has other sizes, or is borrowed itself"
+        freq, self.rot_mag = rotary_frequencies(rot_dims, rot_base, rot_scaling) if rot_dims else ([], 1.0)
+        self.rot_halves = bool(rot_halves)
+        self.register_buffer("rot_freq", torch.tensor(freq, dtype=torch.float32) if rot_dims else None, persistent=False)
+        self.kv_col = q_rank if source is None else -1
+        self.g_col = q_rank + (kv_rank + rot_dim if source is None else 0)
+        self.in_w = _param(self.g_col + (heads if gated else 0), width)
+        self.q_norm, self.uq = _param(q_rank), _param(heads * (dim + rot_dim), q_rank)
+        self.kv_norm = _param(kv_rank) if source is None else None
+        self.uk, self.uv = _param(heads, dim, kv_rank), _param(heads, vdim, kv_rank)
+        self.o_w = _param(width, heads * vdim)
+        self.k_cache = self.v_cache = None            # [pages * block_size, 1, kv_rank + rot_dim] / [.., 1, kv_rank], from the runner
+
+    def kv_shapes(self):
+        """Per-token shapes of this layer's pages: the row [latent | rotated key part] and the latent again as the value (the
+        kernels read values page-transposed). None: the layer reads another layer's pages."""
+        return None if self._source else ((1, self.r + self.dr), (1, self.r))
+
+    def named_loaders(self) -> dict:
+        out = {"dq": _copy_into(self.in_w[:self.qr]), "dq.norm": _copy_into(self.q_norm), "uq": _copy_into(self.uq),
+               "uk": _copy_into(self.uk.view(self.H * self.d, self.r)), "uv": _copy_into(self.uv.view(self.H * self.dv, self.r)),
+               "o": _copy_into(self.o_w)}
+        if not self._source:
+            out.update({"dkv": _copy_into(self.in_w[self.qr:self.g_col]), "dkv.norm": _copy_into(self.kv_norm)})
+        if self.gated:
+            out["g"] = _copy_into(self.in_w[self.g_col:])
+        return out
+
+    def forward(self, xh: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        ctx = get_context()
+        n, H, d, dr, dv, r = xh.shape[0], self.H, self.d, self.dr, self.dv, self.r
+        owner = self._source[0] if self._source else self
+        rot = ops_seq.Rotation(self.rot_freq, self.rot_halves, self.rot_mag) if self.rot_freq is not None else None
+        proj = F.linear(xh, self.in_w)
+        cq = torch.empty(n, self.qr, dtype=xh.dtype, device=xh.device)
+        ops_seq.latent_prep(proj, 0, self.qr, self.q_norm, cq, self.eps, self.kv_col, r, dr, self.kv_norm, positions, rot,
+                            owner.block_size, ctx.slot_mapping, owner.k_cache, owner.v_cache)
+        q = F.linear(cq, self.uq).view(n, H, d + dr)
+        qf = torch.empty(n, H, r + dr, dtype=xh.dtype, device=xh.device)
+        torch.bmm(q[:, :, :d].transpose(0, 1), self.uk, out=qf[:, :, :r].transpose(0, 1))          # W_uk^T q per head
+        ops_seq.rotate_heads(q[:, :, d:], qf[:, :, r:], positions, rot)
+        lat = torch.empty(n, H * r, dtype=xh.dtype, device=xh.device)
+        ops_seq.window_attn(qf.view(n, H * (r + dr)), None, self.eps, proj[:, self.g_col:] if self.gated else None, owner.k_cache,
+                            owner.v_cache, ctx.block_tables, owner.block_size, ctx.portions, H, 1, r + dr, r, self.scale, self.window,
+                            lat, gate_per_head=True)
+        out = torch.empty(n, H, dv, dtype=xh.dtype, device=xh.device)
+        torch.bmm(lat.view(n, H, r).transpose(0, 1), self.uv.transpose(1, 2), out=out.transpose(0, 1))   # W_uv on the latent output
+        return F.linear(out.view(n, H * dv), self.o_w)
 
 
 class LightningMixer(nn.Module):
@@ -317,15 +416,18 @@ class RoutedExperts(nn.Module):
     (`shared_ff`) runs for every token, times sigmoid(w_sg . h). The router's matrix carries w_sg as its last row."""
 
     def __init__(self, width: int, experts: int, ff: int, top: int, scale: float = 1.0, identity: int = 0, group_count: int = 1,
-                 group_keep: int = 1, shared_ff: int = 0):
+                 group_keep: int = 1, shared_ff: int = 0, gated: bool = True, sigmoid: bool = False, renorm: bool = True):
+        """gated False: an expert is W_down max(W_up h, 0)^2 (checkpoint names e<i>.up / e<i>.down). sigmoid: scores are each
+        entry's own sigmoid instead of a softmax over the entries. renorm False: the chosen scores are the weights as they are."""
         super().__init__()
+        self.gated, self.sigmoid, self.renorm = bool(gated), bool(sigmoid), bool(renorm)
         self.E, self.ident, self.ff, self.top, self.scale = experts, identity, ff, top, float(scale)
         self.count, self.keep, self.shared_ff = group_count, group_keep, shared_ff
         total = experts + identity
         assert total % group_count == 0 and 1 <= group_keep <= group_count and top <= group_keep * (total // group_count)
         self.router = _param(total + (1 if shared_ff else 0), width, dtype=torch.float32)
         self.correction = _param(total, dtype=torch.float32)
-        self.w_gu, self.w_down = _param(experts, 2 * ff, width), _param(experts, width, ff)
+        self.w_gu, self.w_down = _param(experts, (2 if gated else 1) * ff, width), _param(experts, width, ff)
         if shared_ff:
             self.s_gu, self.s_down = _param(2 * shared_ff, width), _param(width, shared_ff)
 
@@ -333,8 +435,11 @@ class RoutedExperts(nn.Module):
         total, ff = self.E + self.ident, self.ff
         out = {"router": _copy_into(self.router[:total]), "correction": _copy_into(self.correction)}
         for e in range(self.E):
-            out[f"e{e}.gate"] = _copy_into(self.w_gu[e, :ff])
-            out[f"e{e}.up"] = _copy_into(self.w_gu[e, ff:])
+            if self.gated:
+                out[f"e{e}.gate"] = _copy_into(self.w_gu[e, :ff])
+                out[f"e{e}.up"] = _copy_into(self.w_gu[e, ff:])
+            else:
+                out[f"e{e}.up"] = _copy_into(self.w_gu[e])
             out[f"e{e}.down"] = _copy_into(self.w_down[e])
         if self.shared_ff:
             sf = self.shared_ff
@@ -346,11 +451,11 @@ class RoutedExperts(nn.Module):
         n, width = xh.shape
         total = self.E + self.ident
         z = F.linear(xh.float(), self.router)                                     # 32-bit, [n, total (+ 1: the shared gate)]
-        ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale)
+        ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale, self.sigmoid, self.renorm)
         per_expert = n * self.top // self.E                 # rows an expert gets on average: the tile height follows it
         plan = ops_seq.moe_plan(ids, self.E, 128 if per_expert >= 256 else (64 if per_expert >= 64 else 16))
         act = torch.empty(plan.cap, self.ff, dtype=xh.dtype, device=xh.device)
-        ops_seq.moe_gemm(xh, self.w_gu, plan, True, act)
+        ops_seq.moe_gemm(xh, self.w_gu, plan, self.gated, act, relu2=not self.gated)
         rows = torch.empty(plan.cap, width, dtype=xh.dtype, device=xh.device)
         ops_seq.moe_gemm(act, self.w_down, plan, False, rows)
         shared = gate = None

@@ -15,7 +15,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 
 SIGNATURES = {
@@ -34,11 +34,14 @@ SIGNATURES = {
     "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _I, _L, _P, _P]),
     "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_window_attn_force_scalar": (None, [_I]),
-    "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
+    "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
                                 _I, _P, _I, _P, _P]),
-    "nvs_add_group_norm": (c_int, [_P, _P, _P, _P, _L, _P, _I, _I, _I, _F, _P, _P]),
+    "nvs_add_group_norm": (c_int, [_P, _P, _F, _P, _P, _L, _P, _I, _I, _I, _F, _I, _P, _P]),
+    "nvs_scale_softcap": (c_int, [_P, _I, _F, _F, _L, _P, _P]),
+    "nvs_latent_prep": (c_int, [_P, _L, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _F, _F, _I, _P, _P, _P, _L, _P]),
+    "nvs_rotate_heads": (c_int, [_P, _L, _I, _P, _L, _I, _I, _I, _I, _P, _P, _I, _I, _F, _L, _P]),
     "nvs_glu_act": (c_int, [_P, _L, _I, _I, _I, _F, _F, _L, _P, _P]),
-    "nvs_moe_route": (c_int, [_P, _L, _P, _L, _I, _I, _I, _I, _F, _P, _P, _P]),
+    "nvs_moe_route": (c_int, [_P, _L, _P, _L, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P]),
     "nvs_moe_rows": (c_int64, [_L, _I, _I]),
     "nvs_moe_plan": (c_int, [_P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "nvs_moe_gemm": (c_int, [_P, _L, _P, _I, _I, _I, _I, _P, _P, _L, _I, _P, _L, _P]),
@@ -239,24 +242,26 @@ def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, 
 
 def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: torch.Tensor | None, k_cache, v_cache,
                 block_tables: torch.Tensor, block_size: int, por: Portions, H: int, G: int, d: int, dv: int, scale: float,
-                window: int, out: torch.Tensor, chunk: int = 0, rot_freq: torch.Tensor | None = None):
+                window: int, out: torch.Tensor, chunk: int = 0, rot_freq: torch.Tensor | None = None, gate_per_head: bool = False):
     """window > 0: the last `window` positions; chunk > 0: the query's own block of `chunk` positions; neither: causal.
-    rot_freq [r / 2] (32-bit): the first r entries of every query head turn in interleaved pairs by position * rot_freq."""
+    rot_freq [r / 2] (32-bit): the first r entries of every query head turn in interleaved pairs by position * rot_freq.
+    gate [n, H * dv], or [n, H] with gate_per_head: out *= sigmoid(gate)."""
     lib = load_library()
     n = por.n
     assert q.shape == (n, H * d) and q.stride(1) == 1 and out.shape == (n, H * dv) and out.is_contiguous()
-    assert gate is None or (gate.shape == (n, H * dv) and gate.stride(1) == 1)
+    assert gate is None or (gate.shape == (n, H if gate_per_head else H * dv) and gate.stride(1) == 1)
     assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and block_tables.shape[0] >= por.nseq
     assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
     _check(lib.nvs_window_attn(_ptr(q), q.stride(0), _ptr(qnorm), eps, _ptr(gate), gate.stride(0) if gate is not None else 0,
-                               _same(q, qnorm, gate, k_cache, v_cache, out), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                               int(gate_per_head), _same(q, qnorm, gate, k_cache, v_cache, out), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                block_tables.stride(0), block_size, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.tseq), por.nseq, n, H,
                                G, d, dv, scale, window, chunk, _ptr(rot_freq), _rotation(rot_freq), _ptr(out), _stream()))
 
 
 def add_group_norm(x: torch.Tensor, w: torch.Tensor | None, groups: int, eps: float, out: torch.Tensor | None,
-                   a: torch.Tensor | None = None, b: torch.Tensor | None = None):
-    """x += a + b (in place; a in the activation type, b 32-bit, both optional), then out = group_rms(x) * w (out None: adds only)."""
+                   a: torch.Tensor | None = None, b: torch.Tensor | None = None, a_mult: float = 1.0, center: bool = False):
+    """x += a_mult * a + b (in place; a in the activation type, b 32-bit, both optional), then out = group_rms(x) * w (out None:
+    adds only); center: every group's mean is taken off first (layer norm without bias)."""
     lib = load_library()
     n, width = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
@@ -265,18 +270,71 @@ def add_group_norm(x: torch.Tensor, w: torch.Tensor | None, groups: int, eps: fl
     assert out is None or (out.shape == x.shape and out.is_contiguous() and w is not None and w.numel() == width)
     ref = out if out is not None else a
     assert ref is not None, "nothing to do"
-    _check(lib.nvs_add_group_norm(_ptr(x), _ptr(a), _ptr(b), None, n, _ptr(w) if out is not None else None, _same(ref, a, w, out), width,
-                                  groups, eps, _ptr(out), _stream()))
+    _check(lib.nvs_add_group_norm(_ptr(x), _ptr(a), a_mult, _ptr(b), None, n, _ptr(w) if out is not None else None, _same(ref, a, w, out),
+                                  width, groups, eps, int(center), _ptr(out), _stream()))
 
 
-def group_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor):
-    """out[r] = group_rms(x[rows[r]]) * w (rows None: row r)."""
+def group_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
+                    center: bool = False):
+    """out[r] = group_rms(x[rows[r]]) * w (rows None: row r); center: as add_group_norm."""
     lib = load_library()
     assert x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == (nrows, x.shape[1])
     assert rows is None or (rows.dtype == torch.int32 and rows.numel() >= nrows)
     assert rows is not None or nrows <= x.shape[0]
-    _check(lib.nvs_add_group_norm(_ptr(x), None, None, _ptr(rows), nrows, _ptr(w), _same(out, w), x.shape[1], groups, eps, _ptr(out),
-                                  _stream()))
+    _check(lib.nvs_add_group_norm(_ptr(x), None, 1.0, None, _ptr(rows), nrows, _ptr(w), _same(out, w), x.shape[1], groups, eps, int(center),
+                                  _ptr(out), _stream()))
+
+
+def scale_softcap(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """32-bit cap * tanh(logits * scale / cap) (cap <= 0: logits * scale)."""
+    lib = load_library()
+    assert logits.is_contiguous()
+    out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    _check(lib.nvs_scale_softcap(_ptr(logits), _code(logits), scale, cap, logits.numel(), _ptr(out), _stream()))
+    return out
+
+
+class Rotation:
+    """How the leading `dims` entries of a vector turn with the position: 32-bit frequencies of the pairs (device), the pairing
+    ((2i, 2i+1), or (i, i + dims / 2) with `halves`) and a factor on cos and sin."""
+    __slots__ = ("freq", "dims", "halves", "mag")
+
+    def __init__(self, freq: torch.Tensor, halves: bool = False, mag: float = 1.0):
+        assert freq.dtype == torch.float32 and freq.is_contiguous()
+        self.freq, self.dims, self.halves, self.mag = freq, 2 * freq.numel(), bool(halves), float(mag)
+
+
+def latent_prep(proj: torch.Tensor, q_col: int, q_rank: int, q_norm: torch.Tensor, cq: torch.Tensor, eps: float, kv_col: int = -1,
+                kv_rank: int = 0, rot_dim: int = 0, kv_norm: torch.Tensor | None = None, pos: torch.Tensor | None = None,
+                rot: Rotation | None = None, block_size: int = 0, slots: torch.Tensor | None = None, k_cache: torch.Tensor | None = None,
+                v_cache: torch.Tensor | None = None):
+    """Norms of the query latent (-> cq [n, q_rank]) and, with kv_col >= 0, of the key/value latent, the rotation of the shared key
+    part and the store of both into the paged cache: k_cache [slots, 1, kv_rank + rot_dim], v_cache [slots, 1, kv_rank] (the
+    latent again, page-transposed like every value cache)."""
+    lib = load_library()
+    n = proj.shape[0]
+    assert proj.stride(1) == 1 and cq.shape == (n, q_rank) and cq.is_contiguous() and q_norm.numel() == q_rank
+    if kv_col >= 0:
+        assert kv_norm.numel() == kv_rank and slots.dtype == torch.int32 and slots.numel() >= n
+        assert pos.dtype == torch.int64 and pos.numel() >= n and pos.is_contiguous()
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[0] % block_size == 0
+        assert tuple(k_cache.shape[1:]) == (1, kv_rank + rot_dim) and tuple(v_cache.shape[1:]) == (1, kv_rank)
+        assert rot is None or (rot.freq.is_cuda and rot.dims <= rot_dim)
+    _check(lib.nvs_latent_prep(_ptr(proj), proj.stride(0), _same(proj, q_norm, cq, kv_norm, k_cache, v_cache), q_col, q_rank, _ptr(q_norm),
+                               _ptr(cq), kv_col, kv_rank, rot_dim, _ptr(kv_norm), _ptr(pos), _ptr(rot.freq) if rot else None,
+                               rot.dims if rot else 0, int(rot.halves) if rot else 0, rot.mag if rot else 1.0, eps, block_size, _ptr(slots),
+                               _ptr(k_cache), _ptr(v_cache), n, _stream()))
+
+
+def rotate_heads(inp: torch.Tensor, out: torch.Tensor, pos: torch.Tensor, rot: Rotation | None):
+    """inp, out [n, H, width] views (unit stride along the last axis): out = inp with the leading rot.dims entries of every head rotated."""
+    lib = load_library()
+    n, H, width = inp.shape
+    assert out.shape == inp.shape and inp.stride(2) == 1 and out.stride(2) == 1 and pos.dtype == torch.int64 and pos.numel() >= n
+    assert rot is None or rot.dims <= width
+    _check(lib.nvs_rotate_heads(_ptr(inp), inp.stride(0), inp.stride(1), _ptr(out), out.stride(0), out.stride(1), _same(inp, out), H, width,
+                                _ptr(pos), _ptr(rot.freq) if rot else None, rot.dims if rot else 0, int(rot.halves) if rot else 0,
+                                rot.mag if rot else 1.0, n, _stream()))
 
 
 def decay_scan(proj: torch.Tensor, v_col: int, k_col: int, q_col: int, decay: torch.Tensor, heads: int, dk: int, dv: int,
@@ -302,15 +360,18 @@ def glu_act(gu: torch.Tensor, ff: int, out: torch.Tensor, kind: int = 0, limit: 
     _check(lib.nvs_glu_act(_ptr(gu), gu.stride(0), _same(gu, out), ff, kind, limit, alpha, n, _ptr(out), _stream()))
 
 
-def moe_route(z: torch.Tensor, total: int, correction: torch.Tensor | None, top: int, count: int, keep: int, scale: float):
-    """z [n, >= total] 32-bit router logits -> (ids [n, top] int32, weights [n, top] 32-bit)."""
+def moe_route(z: torch.Tensor, total: int, correction: torch.Tensor | None, top: int, count: int, keep: int, scale: float,
+              sigmoid: bool = False, renorm: bool = True):
+    """z [n, >= total] 32-bit router logits -> (ids [n, top] int32, weights [n, top] 32-bit). Scores are a softmax over the entries,
+    or with `sigmoid` every entry's own sigmoid; weights are the chosen scores, divided by their sum with `renorm`, times scale."""
     lib = load_library()
     n = z.shape[0]
     assert z.dtype == torch.float32 and z.stride(1) == 1 and z.shape[1] >= total
     assert correction is None or (correction.dtype == torch.float32 and correction.numel() == total and correction.is_contiguous())
     ids = torch.empty(n, top, dtype=torch.int32, device=z.device)
     wts = torch.empty(n, top, dtype=torch.float32, device=z.device)
-    _check(lib.nvs_moe_route(_ptr(z), z.stride(0), _ptr(correction), n, total, top, count, keep, scale, _ptr(ids), _ptr(wts), _stream()))
+    _check(lib.nvs_moe_route(_ptr(z), z.stride(0), _ptr(correction), n, total, top, count, keep, scale, int(sigmoid), int(renorm), _ptr(ids),
+                             _ptr(wts), _stream()))
     return ids, wts
 
 
@@ -332,13 +393,15 @@ def moe_plan(ids: torch.Tensor, experts: int, tm: int) -> MoePlan:
     return p
 
 
-def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, glu: bool, out: torch.Tensor):
-    """glu: w [experts, 2 nout, K], rows gathered by token, out = silu(gate) * up; else w [experts, nout, K], x holds the planned rows."""
+def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, glu: bool, out: torch.Tensor, relu2: bool = False):
+    """glu: w [experts, 2 nout, K], rows gathered by token, out = silu(gate) * up; relu2: w [experts, nout, K], rows gathered by
+    token, out = max(w x, 0)^2; neither: w [experts, nout, K], x holds the planned rows."""
     lib = load_library()
+    assert not (glu and relu2)
     nout, K = (w.shape[1] // 2 if glu else w.shape[1]), w.shape[2]
     assert w.is_contiguous() and x.stride(1) == 1 and x.shape[1] == K and out.shape == (plan.cap, nout) and out.stride(1) == 1
-    assert glu or x.shape[0] == plan.cap
-    _check(lib.nvs_moe_gemm(_ptr(x), x.stride(0), _ptr(w), _same(x, w, out), int(glu), nout, K, _ptr(plan.tile_expert), _ptr(plan.row_token),
+    assert glu or relu2 or x.shape[0] == plan.cap
+    _check(lib.nvs_moe_gemm(_ptr(x), x.stride(0), _ptr(w), _same(x, w, out), 1 if glu else (2 if relu2 else 0), nout, K, _ptr(plan.tile_expert), _ptr(plan.row_token),
                             plan.cap, plan.tm, _ptr(out), out.stride(0), _stream()))
 
 

@@ -58,12 +58,24 @@ def _nokipel_build(config, dtype=None):
     return NokipelForCausalLM(config, dtype)
 
 
+def _pefazen_config(path: str, raw: dict):
+    from .pefazen import PefazenConfig
+    return PefazenConfig(raw)
+
+
+def _pefazen_build(config, dtype=None):
+    from .pefazen import PefazenForCausalLM
+    return PefazenForCausalLM(config, dtype)
+
+
 REGISTRY: dict[str, ModelSpec] = {
     "Qwen3ForCausalLM": ModelSpec("Qwen3ForCausalLM", _qwen3_config, _qwen3_build),
     "Qwen2ForCausalLM": ModelSpec("Qwen2ForCausalLM", _qwen3_config, _qwen3_build),      # same module tree, biased qkv, no q/k norm
     "Foduzen": ModelSpec("Foduzen", _foduzen_config, _foduzen_build, stateful=True, block_multiple=16,
                          dtypes=("bfloat16", "float32")),
     "Nokipel": ModelSpec("Nokipel", _nokipel_config, _nokipel_build, stateful=True, block_multiple=16,
+                         dtypes=("bfloat16", "float32")),
+    "Pefazen": ModelSpec("Pefazen", _pefazen_config, _pefazen_build, stateful=True, block_multiple=16,
                          dtypes=("bfloat16", "float32")),
 }
 
