@@ -29,9 +29,9 @@ driver's fields it carries
                  race keys with the draws replayed (a by-product of the cpu_baseline leg: the timed
                  oracle pass is teacher-forced with the engine's tokens).
 
-`python bench.py --compare-families [--families nokipel,foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a line
-of its own (metric "family_compare"): prefill and decode throughput of the Nokipel and Foduzen families at layer sizes of real
-models beside Qwen3 at equal width and depth. The default command above is unchanged by it.
+`python bench.py --compare-families [--families pefazen,nokipel,foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a
+line of its own (metric "family_compare"): prefill and decode throughput of the Pefazen, Nokipel and Foduzen families at layer
+sizes of real models beside Qwen3 at equal width and depth. The default command above is unchanged by it.
 """
 from __future__ import annotations
 
@@ -89,9 +89,9 @@ def parse():
     ap.add_argument("--kv-cache-dtype", default="bf16", choices=["bf16", "fp8"],
                     help="fp8: opt-in OCP e4m3 KV cache (outside the reference's numerics; never the headline)")
     ap.add_argument("--compare-families", action="store_true",
-                    help="instead of the headline workload: prefill and decode throughput of the Nokipel and Foduzen families at "
+                    help="instead of the headline workload: prefill and decode throughput of the Pefazen, Nokipel and Foduzen families at "
                          "layer sizes of real models (random weights) beside Qwen3 models of equal width / depth, one JSON line")
-    ap.add_argument("--families", default="nokipel,foduzen,qwen3", help="with --compare-families: which of the three to run")
+    ap.add_argument("--families", default="pefazen,nokipel,foduzen,qwen3", help="with --compare-families: which of the four to run")
     ap.add_argument("--sizes", default="1k,4k", help="with --compare-families: layer sizes to run (1k, 4k)")
     return ap.parse_args()
 
@@ -126,6 +126,28 @@ def nokipel_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, 
             "norm": {"eps": 1e-6, "groups": 1}, "vocab": vocab, "width": width}
 
 
+def pefazen_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, vocab: int) -> dict:
+    """Layers of a real model's size: heads of 128 unrotated + 64 rotated query / key entries and 128 value entries over a latent
+    of 192 (+ 64 rotated: a cached row of 256, the longest the matrix-core attention takes), a query latent of 3/8 of the width;
+    windowed gated layers (1,024 positions) and causal layers with scaled frequencies alternate, the third layer reads the first
+    one's cache; every layer has 32 experts of a quarter of the dense width, 4 chosen."""
+    def mixer(**kw):
+        return dict({"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 3 * width // 8, "kv_rank": 192, "scale": 192 ** -0.5}, **kw)
+    mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}}
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            m = mixer(mask={"size": 1024}, rot={"dims": 64, "base": 10000.0})
+            if i == 2:
+                m["kv_from"] = 0
+            out.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+        else:
+            rot = {"dims": 64, "base": 500000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+            out.append({"type": "latent_attention_2", "mixer": mixer(rot=rot), "mlp": mlp})
+    return {"architecture": "Pefazen", "layers": out, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width, "residual_mult": 1.0,
+            "logit_scale": 1.0, "logit_softcap": 30.0}
+
+
 FAMILY_SIZES = {   # name: (width, ff, heads, kv heads, layers, the Qwen3 shape of the same width / depth)
     "1k": (1024, 3072, 16, 8, 4, "qwen3-0.6b-4l"),
     "4k": (4096, 12288, 32, 8, 2, "qwen3-8b-2l"),
@@ -147,8 +169,8 @@ def compare_families(args) -> dict:
         width, ff, heads, kv, layers, qname = FAMILY_SIZES[size]
         for family in args.families.split(","):
             path = os.path.join(tempfile.gettempdir(), f"nvl_cmp_{family}_{size}")
-            if family in ("foduzen", "nokipel"):
-                raw = (foduzen_config if family == "foduzen" else nokipel_config)(width, ff, heads, kv, layers, vocab)
+            if family in ("foduzen", "nokipel", "pefazen"):
+                raw = {"foduzen": foduzen_config, "nokipel": nokipel_config, "pefazen": pefazen_config}[family](width, ff, heads, kv, layers, vocab)
                 os.makedirs(path, exist_ok=True)
                 with open(os.path.join(path, "config.json"), "w") as fh:
                     json.dump(raw, fh)

@@ -117,13 +117,13 @@ int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, c
                       int block_size, const int32_t* slots, const int64_t* pos, const float* rot_freq, int rot_dims, int64_t n,
                       void* k_cache, void* v_cache, void* stream);
 
-/* Locally masked softmax attention over the paged cache, one query per token row, any d, dv <= 256.
+/* Locally masked softmax attention over the paged cache, one query per token row, any d, dv <= 1024.
  * q [n, H, d] (row stride q_stride), RMS-normed per head with qnorm [d] here (NULL: none), then rotated like the keys
  * (rot_dims, rot_freq; 0: not). Token t of portion s sits at position p = ctx0[s] + (t - cu_q[s]) and sees keys j with
  * 0 <= p - j < window (window > 0), or the keys j <= p of its own block, floor(j / chunk) == floor(p / chunk) (chunk > 0; blocks
  * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
  * gate_stride: out *= sigmoid(gate); with gate_per_head != 0 the gate is [n, H], one entry for all columns of a head. out [n, H*dv] `dtype`.
- * bf16 with d % 8 == 0 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
+ * bf16 with d % 8 == 0, d and dv <= 256 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
  * second product as bf16); everything else, and every float32 call, takes the scalar kernel (one wavefront per query). */
 int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_per_head, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,

@@ -7,7 +7,7 @@
 
 namespace {
 
-constexpr int MAX_HEAD = 256;
+constexpr int MAX_HEAD = 1024;      // scalar kernels (CH = 4 or 16 chunks of 64 entries per head); the matrix-core kernels take up to 256
 
 // first key position the query at position p sees (both masks are monotone in p, which the tile bounds below rely on)
 __device__ __forceinline__ int vis_lo(int p, int window, int chunk) {
@@ -17,7 +17,7 @@ __device__ __forceinline__ int vis_lo(int p, int window, int chunk) {
 }
 
 // one wavefront per (token, kv head)
-template <typename T>
+template <typename T, int CH>
 __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restrict__ v, int64_t stride, const T* __restrict__ knorm,
                                      float eps, int G, int d, int dv, int block_size, const int32_t* __restrict__ slots,
                                      const int64_t* __restrict__ pos, const float* __restrict__ rot_freq, int rot_dims,
@@ -27,10 +27,10 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
   const int64_t slot = slots[t];
   if (slot < 0) return;
   const T* kp = k + t * stride + (int64_t)g * d;
-  float kv[MAX_HEAD / 64];
+  float kv[CH];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < MAX_HEAD / 64; ++i) {
+  for (int i = 0; i < CH; ++i) {
     const int c = lane + 64 * i;
     kv[i] = c < d ? ldf(kp + c) : 0.f;
     ss += kv[i] * kv[i];
@@ -40,7 +40,7 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
   T* kc = k_cache + (slot * G + g) * d;
   const float pf = rot_dims > 0 ? (float)pos[t] : 0.f;
 #pragma unroll
-  for (int i = 0; i < MAX_HEAD / 64; ++i) {
+  for (int i = 0; i < CH; ++i) {
     const int c = lane + 64 * i;
     float val = (knorm && c < d) ? kv[i] * r * ldf(knorm + c) : kv[i];
     // rotation of the pair (2i, 2i+1): the partner sits in the neighbouring lane
@@ -61,14 +61,14 @@ __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restric
 
 // one wavefront per (token, query head). Keys go in rounds of 64 (one per lane): score, running maximum, weights into LDS,
 // then every lane accumulates its value columns over the round's keys.
-template <typename T>
+template <typename T, int CH>
 __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, const T* __restrict__ qnorm, float eps,
                                    const T* __restrict__ gate, int64_t gate_stride, int gate_w, const T* __restrict__ k_cache,
                                    const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int64_t bt_stride,
                                    int block_size, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
                                    const int32_t* __restrict__ tseq, int H, int G, int d, int dv, float scale, int window, int chunk,
                                    const float* __restrict__ rot_freq, int rot_dims, T* __restrict__ out) {
-  __shared__ float qs[MAX_HEAD];
+  __shared__ float qs[CH * 64];
   __shared__ float ps[64];
   __shared__ int64_t slot_s[64];                    // element offset of (token, column 0) in the page-transposed V cache
   const int64_t t = blockIdx.x;
@@ -79,17 +79,17 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
   // query (+ norm) into LDS
   {
     const T* qp = q + t * q_stride + (int64_t)h * d;
-    float qv[MAX_HEAD / 64];
+    float qv[CH];
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < MAX_HEAD / 64; ++i) {
+    for (int i = 0; i < CH; ++i) {
       const int c = lane + 64 * i;
       qv[i] = c < d ? ldf(qp + c) : 0.f;
       ss += qv[i] * qv[i];
     }
     const float r = qnorm ? rsqrtf(wave_sum(ss) / (float)d + eps) : 1.f;
 #pragma unroll
-    for (int i = 0; i < MAX_HEAD / 64; ++i) {
+    for (int i = 0; i < CH; ++i) {
       const int c = lane + 64 * i;
       float val = (qnorm && c < d) ? qv[i] * r * ldf(qnorm + c) : qv[i];
       const float other = __shfl_xor(val, 1, 64);   // rotation of the pair (2i, 2i+1)
@@ -105,9 +105,9 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
   const int64_t lo = vis_lo((int)pos, window, chunk);
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
   float m = -INFINITY, l = 0.f;
-  float acc[MAX_HEAD / 64];
+  float acc[CH];
 #pragma unroll
-  for (int i = 0; i < MAX_HEAD / 64; ++i) acc[i] = 0.f;
+  for (int i = 0; i < CH; ++i) acc[i] = 0.f;
   for (int64_t j0 = lo; j0 <= pos; j0 += 64) {
     const int64_t j = j0 + lane;
     const bool live = j <= pos;
@@ -133,7 +133,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
     __syncthreads();
     const int cnt = (int)((pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64);
 #pragma unroll
-    for (int i = 0; i < MAX_HEAD / 64; ++i) {
+    for (int i = 0; i < CH; ++i) {
       const int c = lane + 64 * i;
       if (c < dv) {
         float a = acc[i] * alpha;
@@ -144,7 +144,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
   }
   const float inv = 1.f / l;
 #pragma unroll
-  for (int i = 0; i < MAX_HEAD / 64; ++i) {
+  for (int i = 0; i < CH; ++i) {
     const int c = lane + 64 * i;
     if (c < dv) {
       float o = acc[i] * inv;
@@ -617,7 +617,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
   int bs_shift = -1;
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == block_size) bs_shift = b;
-  if constexpr (64 * (32 * DK + 8) * 2 + 16 * DVB * 72 * 2 <= 65536) {
+  if constexpr (64 * (32 * DK + 8) * 2 + 16 * DVB * 72 * 2 <= 160 * 1024) {      // (every size does: gfx950 has 160 KB of LDS per CU)
     if (!g_no_lds) {
       const int hpg = H / G, hw = hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
       const int bq = (4 / hw) * 16 * QT;
@@ -668,9 +668,14 @@ extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, i
   NVS_REQUIRE(G > 0 && G <= 65535 && d > 0 && d <= MAX_HEAD && dv > 0 && dv <= MAX_HEAD && n >= 0 && block_size > 0,
               "nvs_knorm_kvstore: G %d d %d dv %d", G, d, dv);
   if (n == 0) return NVS_OK;
-  NVS_DISPATCH(dtype, knorm_kvstore_kernel<T><<<dim3((unsigned)n, G), dim3(64), 0, (hipStream_t)stream>>>(
-                          (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, pos, rot_freq, rot_dims, (T*)k_cache,
-                          (T*)v_cache));
+  if (d <= 256 && dv <= 256)
+    NVS_DISPATCH(dtype, knorm_kvstore_kernel<T, 4><<<dim3((unsigned)n, G), dim3(64), 0, (hipStream_t)stream>>>(
+                            (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, pos, rot_freq, rot_dims,
+                            (T*)k_cache, (T*)v_cache));
+  else
+    NVS_DISPATCH(dtype, knorm_kvstore_kernel<T, 16><<<dim3((unsigned)n, G), dim3(64), 0, (hipStream_t)stream>>>(
+                            (const T*)k, (const T*)v, stride, (const T*)knorm, eps, G, d, dv, block_size, slots, pos, rot_freq, rot_dims,
+                            (T*)k_cache, (T*)v_cache));
   return nvs_check_launch("nvs_knorm_kvstore");
 }
 
@@ -687,7 +692,7 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
               "nvs_window_attn: H %d G %d d %d dv %d block %d", H, G, d, dv, block_size);
   if (n == 0 || nseq == 0) return NVS_OK;
   const int gate_w = gate_per_head ? 1 : dv;         // gate entries per head: one for the whole head, or one per value column
-  if (dtype == NVS_BF16 && d % 8 == 0 && block_size % 8 == 0 && !g_force_scalar) {
+  if (dtype == NVS_BF16 && d % 8 == 0 && d <= 256 && dv <= 256 && block_size % 8 == 0 && !g_force_scalar) {
     const int dk = d <= 64 ? 2 : (d <= 128 ? 4 : 8), dvb = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
 #define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
   if (dk == DK && dvb == DVB)                                                                                                   \
@@ -698,8 +703,15 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
 #undef NVS_MFMA_CASE
     return nvs_check_launch("nvs_window_attn (matrix cores)");
   }
-  NVS_DISPATCH(dtype, window_attn_kernel<T><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
-                          (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache, (const T*)v_cache,
-                          block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, (T*)out));
+  if (d <= 256 && dv <= 256)
+    NVS_DISPATCH(dtype, window_attn_kernel<T, 4><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
+                            (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache,
+                            (const T*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq,
+                            rot_dims, (T*)out));
+  else                                               // heads of up to 1024 entries: the same kernel with 16 entries per lane
+    NVS_DISPATCH(dtype, window_attn_kernel<T, 16><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
+                            (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache,
+                            (const T*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq,
+                            rot_dims, (T*)out));
   return nvs_check_launch("nvs_window_attn");
 }

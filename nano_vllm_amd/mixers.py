@@ -153,7 +153,8 @@ class LatentAttentionMixer(nn.Module):
         super().__init__()
         rot_dims = rot_dim if rot_dims is None else int(rot_dims)
         assert rot_dims % 2 == 0 and 0 <= rot_dims <= rot_dim
-        assert kv_rank + rot_dim <= 256, f"latent row of {kv_rank} + {rot_dim} entries: the attention kernels take up to 256"
+        # (rows of up to 256 entries run on the matrix cores in bf16, longer ones on the scalar kernel)
+        assert kv_rank + rot_dim <= 1024, f"latent row of {kv_rank} + {rot_dim} entries: the attention kernels take up to 1024"
         self.H, self.d, self.dr, self.dv, self.qr, self.r = heads, dim, rot_dim, vdim, q_rank, kv_rank
         self.scale, self.eps, self.window, self.gated, self.block_size = float(scale), eps, int(window), bool(gated), block_size
         self._source = (source,) if source is not None else ()          # (a tuple: not a submodule of this layer)

@@ -119,7 +119,7 @@ def route(z: np.ndarray, correction: np.ndarray, top: int) -> tuple[np.ndarray, 
     return ids, wts
 
 
-def routed_experts(h: np.ndarray, w: dict, mlp: dict, forced_ids: np.ndarray | None = None) -> np.ndarray:
+def routed_experts(h: np.ndarray, w: dict, mlp: dict) -> np.ndarray:
     """Mixture of experts W_down relu(W_up h)^2; weights are not renormalised."""
     E, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     ids, wts = route(h @ f64(w["router"]).T, f64(w["correction"]), top)
@@ -160,3 +160,23 @@ def forward(raw: dict, tensors: dict, tokens, trace: list | None = None) -> np.n
     z = layer_norm(x, f64(tensors["final.norm"]), eps) @ f64(tensors["head"]).T * float(raw.get("logit_scale", 1.0))
     cap = float(raw.get("logit_softcap") or 0.0)
     return cap * np.tanh(z / cap) if cap > 0 else z
+
+
+class Model:
+    """A checkpoint directory read into float64 (config.json + model.safetensors)."""
+
+    def __init__(self, cfg: dict, tensors: dict):
+        self.cfg, self.tensors = cfg, {k: f64(v) for k, v in tensors.items()}
+
+    @classmethod
+    def load(cls, path: str) -> "Model":
+        import json
+        import os
+
+        from safetensors.torch import load_file
+        with open(os.path.join(path, "config.json")) as fh:
+            cfg = json.load(fh)
+        return cls(cfg, load_file(os.path.join(path, "model.safetensors")))
+
+    def run(self, tokens, trace: list | None = None) -> np.ndarray:
+        return forward(self.cfg, self.tensors, tokens, trace)

@@ -246,3 +246,77 @@ def test_nokipel_checkpoint_names_loaders_and_weights_shared_between_runs():
     assert torch.equal(moe.w_gu[2, 10:], tensors["l1.mlp.e2.up"].float()) and moe.correction.dtype == torch.float32
     with pytest.raises(AssertionError):
         loaders["embed"](torch.zeros(3, 3))
+
+
+# ---- Pefazen: configuration, borrowed caches, scaled rotation table, checkpoint names (no GPU) ----------------------------
+def pfz_raw():
+    def mixer(H, d, dr, dv, qr, r, **kw):
+        return dict({"heads": H, "dim": d, "rot_dim": dr, "vdim": dv, "q_rank": qr, "kv_rank": r, "scale": 0.2}, **kw)
+    moe = {"kind": "moe", "expert": {"ff": 10}, "router": {"experts": 3, "top": 2}}
+    a = {"type": "latent_attention", "mixer": mixer(2, 6, 4, 8, 5, 12, mask={"size": 7}, rot={"dims": 4, "base": 100.0}), "mlp": moe}
+    b = {"type": "latent_attention_2", "mlp": None,
+         "mixer": mixer(3, 4, 8, 6, 7, 10, rot={"dims": 8, "base": 10000.0, "scaling": {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0}})}
+    c = {"type": "latent_attention", "mixer": mixer(4, 2, 4, 2, 3, 12, mask={"size": 3}, rot={"dims": 4, "base": 100.0}, kv_from=0), "mlp": moe}
+    return {"architecture": "Pefazen", "layers": [a, b, c], "norm": {"eps": 1e-5}, "vocab": 29, "width": 16, "residual_mult": 0.5,
+            "logit_scale": 0.125, "logit_softcap": 20.0}
+
+
+def test_pefazen_registry_and_config_checks(tmp_path):
+    from nano_vllm_amd.registry import REGISTRY, resolve
+    (tmp_path / "config.json").write_text(json.dumps(pfz_raw()))
+    spec, cfg = resolve(str(tmp_path))
+    assert spec is REGISTRY["Pefazen"] and spec.stateful and set(spec.dtypes) == {"bfloat16", "float32"}
+    assert (cfg.vocab_size, cfg.hidden_size, cfg.residual_mult, cfg.logit_scale, cfg.logit_softcap) == (29, 16, 0.5, 0.125, 20.0)
+    cases = [(lambda r: r["layers"][0].update(type="lstm"), "mixer type"), (lambda r: r["layers"][0].update(mlp={"kind": "dense"}), "feed-forward kind"),
+             (lambda r: r["layers"][2]["mixer"].update(kv_from=2), "kv_from"), (lambda r: r["layers"][1]["mixer"].update(kv_from=2), "kv_from"),
+             (lambda r: r["layers"][2]["mixer"].update(kv_rank=14), "latent sizes")]
+    for change, msg in cases:
+        raw = pfz_raw()
+        change(raw)
+        (tmp_path / "config.json").write_text(json.dumps(raw))
+        with pytest.raises(ValueError, match=msg):
+            resolve(str(tmp_path))
+
+
+def test_pefazen_checkpoint_names_loaders_and_the_borrowed_cache():
+    """Every tensor the synthetic checkpoint writes has a loader in the model and the other way round; the layer that reads
+    another layer's cache has no down projection for keys and values and asks the engine for no pages."""
+    from nano_vllm_amd.pefazen import PefazenConfig, PefazenForCausalLM, random_tensors, tensor_shapes
+    raw = pfz_raw()
+    model = PefazenForCausalLM(PefazenConfig(raw), torch.float32, block_size=16)
+    loaders, shapes = model.named_loaders(), tensor_shapes(raw)
+    assert set(loaders) == set(shapes) and "l2.mix.dkv" not in shapes and "l1.mix.g" not in shapes and "l1.norm2" not in shapes
+    tensors = random_tensors(raw, seed=3)
+    with torch.no_grad():
+        for name, t in tensors.items():
+            assert tuple(t.shape) == tuple(shapes[name]) and t.dtype == torch.bfloat16
+            loaders[name](t)
+    a, b, c = (layer.mixer for layer in model.layers)
+    assert a.kv_shapes() == ((1, 16), (1, 12)) and b.kv_shapes() == ((1, 18), (1, 10)) and c.kv_shapes() is None
+    assert c._source[0] is a and len(list(c.parameters())) == len(list(a.parameters())) - 1
+    assert sum(p.numel() for p in model.parameters()) == sum(int(torch.tensor(s).prod()) for s in shapes.values())
+    # fused in-projection: [query latent | key/value latent + rotated key part | gate]
+    assert a.in_w.shape == (5 + 16 + 2, 16) and b.in_w.shape == (7 + 18, 16) and c.in_w.shape == (3 + 4, 16)
+    assert torch.equal(a.in_w[5:21], tensors["l0.mix.dkv"].float()) and torch.equal(c.in_w[3:], tensors["l2.mix.g"].float())
+    assert torch.equal(a.uk.view(12, 12), tensors["l0.mix.uk"].float()) and torch.equal(b.uv[2], tensors["l1.mix.uv"].float()[12:18])
+    assert (a.window, b.window, c.window) == (7, 0, 3) and (a.gated, b.gated) == (True, False) and (a.rot_halves, b.rot_halves) == (False, True)
+    assert a.rot_mag == 1.0 and a.rot_freq.tolist() == [1.0, pytest.approx(0.1)]
+    moe = model.layers[0].mlp
+    assert (moe.gated, moe.sigmoid, moe.renorm) == (False, True, False) and moe.w_gu.shape == (3, 10, 16) and model.layers[1].mlp is None
+
+
+def test_scaled_rotation_table_blends_between_the_two_marks():
+    """factor 4 over 64 original positions: pairs turning more than 8 times keep their frequency, pairs turning less than once
+    have it divided by 4, the pairs between blend linearly in the pair index; cos and sin grow by 0.1 ln 4 + 1."""
+    import math
+    from nano_vllm_amd.mixers import rotary_frequencies
+    base, dims = 10000.0, 8
+    freq, mag = rotary_frequencies(dims, base, {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0})
+    plain = [base ** (-2 * i / dims) for i in range(dims // 2)]
+    assert mag == pytest.approx(0.1 * math.log(4.0) + 1.0)
+    lo = math.floor(dims * math.log(64 / (2 * math.pi * 8.0)) / (2 * math.log(base)))        # 0
+    hi = math.ceil(dims * math.log(64 / (2 * math.pi * 1.0)) / (2 * math.log(base)))         # 2
+    assert (lo, hi) == (0, 2)
+    assert freq[0] == pytest.approx(plain[0]) and freq[1] == pytest.approx(plain[1] * (0.5 / 4 + 0.5))
+    assert freq[2] == pytest.approx(plain[2] / 4) and freq[3] == pytest.approx(plain[3] / 4)
+    assert rotary_frequencies(dims, base) == (plain, 1.0)
