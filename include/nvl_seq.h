@@ -123,7 +123,8 @@ int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, c
  * 0 <= p - j < window (window > 0), or the keys j <= p of its own block, floor(j / chunk) == floor(p / chunk) (chunk > 0; blocks
  * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
  * gate_stride: out *= sigmoid(gate); with gate_per_head != 0 the gate is [n, H], one entry for all columns of a head. out [n, H*dv] `dtype`.
- * bf16 with d % 8 == 0, d and dv <= 256 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront; the weights enter the
+ * bf16 with d % 8 == 0, d and dv <= 256 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront — 16 positions of
+ * one head, or in steps of single tokens with 8 or more query heads per kv head 16 heads at one position; the weights enter the
  * second product as bf16); everything else, and every float32 call, takes the scalar kernel (one wavefront per query). */
 int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_per_head, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
@@ -182,7 +183,8 @@ int nvs_rotate_heads(const void* in, int64_t in_stride, int in_head, void* out, 
                      void* stream);
 
 /* Tests and A/B runs: 1 routes bf16 calls through the scalar kernel too; 2 keeps the matrix-core kernel but without sharing
- * K / V tiles through LDS; 0 restores the defaults. */
+ * K / V tiles through LDS; 3 keeps the LDS kernel but never packs heads into the query tiles of single-token steps; 0 restores
+ * the defaults. */
 void nvs_window_attn_force_scalar(int on);
 
 #ifdef __cplusplus

@@ -173,6 +173,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 int g_no_lds = 0;          // tests / A-B: 1 keeps every wavefront on its own operand loads (no LDS sharing)
+int g_packed_heads = 1;    // tests / A-B: 0 never packs heads into the query tiles
 
 template <int DK, int DVB, int QT>     // d <= 32 DK, dv <= 16 DVB, QT tiles of 16 queries per wavefront (they share every K / V load)
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
@@ -388,9 +389,14 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t Ks[64][KP];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * DVB][VP];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, qi = lane & 15, gq = lane >> 4;
-  const int hpg = H / G, chunks = hpg / hw;
-  const int g = blockIdx.y / chunks, h = g * hpg + (blockIdx.y % chunks) * hw + (wave % hw);
-  const int tq = 4 / hw, BQ = tq * QW;             // query tiles and queries of the workgroup
+  // hw == 0 ("packed", QT == 1): the workgroup serves ONE token and the rows of a wavefront's query tile are 16 HEADS of the kv
+  // group at that token (64 heads per workgroup) — for steps of single tokens with many query heads per kv head, where a
+  // tile of 16 consecutive positions would hold one query.
+  const bool packed = hw == 0;
+  const int hpg = H / G, chunks = packed ? (hpg + 63) / 64 : hpg / hw;
+  const int g = blockIdx.y / chunks;
+  const int hl0 = packed ? (blockIdx.y % chunks) * 64 + wave * 16 : (blockIdx.y % chunks) * hw + (wave % hw);   // the wavefront's first head in the group
+  const int BQ = packed ? 1 : (4 / hw) * QW;       // queries (positions) of the workgroup
   int btile = blockIdx.x, s = 0, len = 0;
   for (; s < nseq; ++s) {
     len = cu_q[s + 1] - cu_q[s];
@@ -400,8 +406,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
   }
   if (s >= nseq) return;                            // the whole workgroup leaves
   const int c0 = ctx0[s];
-  const int rel0 = btile * BQ + (wave / hw) * QW;   // this wavefront's first query inside the portion (may lie beyond its end)
-  const int p_first = c0 + rel0, p_hi = c0 + rel0 + QW - 1;
+  const int rel0 = packed ? btile : btile * BQ + (wave / hw) * QW;   // this wavefront's first query inside the portion (may lie beyond its end)
+  const int p_first = c0 + rel0, p_hi = packed ? p_first : c0 + rel0 + QW - 1;
+  const bool idle = packed ? hl0 >= hpg : rel0 >= len;               // a wavefront without queries only helps to load
   const int b_first = c0 + btile * BQ;
   const int b_last = c0 + (btile * BQ + BQ - 1 < len ? btile * BQ + BQ - 1 : len - 1);
   const int bs_mask = block_size - 1;
@@ -410,16 +417,18 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
   bf16x8_t qb[QT][DK];
   bool valid_q[QT];
   int64_t row[QT];
-  int pos[QT];
+  int pos[QT], hq[QT];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    const int rel = rel0 + t * 16 + qi;
-    valid_q[t] = rel < len;
-    row[t] = (int64_t)cu_q[s] + (valid_q[t] ? rel : len - 1);
+    const int rel = packed ? rel0 : rel0 + t * 16 + qi;
+    const int hl = packed ? hl0 + qi : hl0;
+    valid_q[t] = rel < len && hl < hpg;
+    hq[t] = g * hpg + (hl < hpg ? hl : hpg - 1);
+    row[t] = (int64_t)cu_q[s] + (rel < len ? rel : len - 1);
     pos[t] = c0 + rel;
     float qv[DK][8];
     float ss = 0.f;
-    const bf16_t* qp = q + row[t] * q_stride + (int64_t)h * d;
+    const bf16_t* qp = q + row[t] * q_stride + (int64_t)hq[t] * d;
 #pragma unroll
     for (int c = 0; c < DK; ++c)
 #pragma unroll
@@ -522,7 +531,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
       lookup(j0 + 128);
     }
     // a wavefront whose queries all lie before the round's tokens (or beyond the portion) has nothing to add
-    if (j0 > p_hi || rel0 >= len || j0 + 63 < lo_first) continue;
+    if (j0 > p_hi || idle || j0 + 63 < lo_first) continue;
     const bool interior = j0 + 63 <= p_first && j0 >= lo_hi;
     f32x4_t sacc[QT][4];
 #pragma unroll
@@ -593,8 +602,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
     ls += __shfl_xor(ls, 32, 64);
     if (!valid_q[t]) continue;
     const float inv = 1.f / ls;
-    bf16_t* op = out + ((int64_t)row[t] * H + h) * dv;
-    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)h * gate_w : nullptr;
+    bf16_t* op = out + ((int64_t)row[t] * H + hq[t]) * dv;
+    const bf16_t* gp = gate ? gate + row[t] * gate_stride + (int64_t)hq[t] * gate_w : nullptr;
 #pragma unroll
     for (int db = 0; db < DVB; ++db)
 #pragma unroll
@@ -619,7 +628,18 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
     if ((1 << b) == block_size) bs_shift = b;
   if constexpr (64 * (32 * DK + 8) * 2 + 16 * DVB * 72 * 2 <= 160 * 1024) {      // (every size does: gfx950 has 160 KB of LDS per CU)
     if (!g_no_lds) {
-      const int hpg = H / G, hw = hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
+      const int hpg = H / G;
+      if constexpr (QT == 1) {
+        // steps of (mostly) single tokens with many query heads per kv head: heads, not positions, fill the query tiles
+        if (hpg >= 8 && 4 * n <= (int64_t)nseq * hpg && g_packed_heads) {
+          window_attn_mfma_lds_kernel<DK, DVB, 1><<<dim3((unsigned)n, (unsigned)(G * ((hpg + 63) / 64))), dim3(256), 0, stream>>>(
+              (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
+              (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq,
+              rot_dims, bs_shift, 0, (bf16_t*)out);
+          return;
+        }
+      }
+      const int hw = hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
       const int bq = (4 / hw) * 16 * QT;
       const int64_t btiles = n / bq + nseq;         // an upper bound: every portion may end with a partial tile
       window_attn_mfma_lds_kernel<DK, DVB, QT><<<dim3((unsigned)btiles, (unsigned)(G * (hpg / hw))), dim3(256), 0, stream>>>(
@@ -657,6 +677,7 @@ static int g_force_scalar = 0;
 extern "C" void nvs_window_attn_force_scalar(int on) {
   g_force_scalar = on == 1;
   g_no_lds = on == 2;
+  g_packed_heads = on != 3;
 }
 
 extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, const void* knorm, float eps, int G, int d,
@@ -693,13 +714,13 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
   if (n == 0 || nseq == 0) return NVS_OK;
   const int gate_w = gate_per_head ? 1 : dv;         // gate entries per head: one for the whole head, or one per value column
   if (dtype == NVS_BF16 && d % 8 == 0 && d <= 256 && dv <= 256 && block_size % 8 == 0 && !g_force_scalar) {
-    const int dk = d <= 64 ? 2 : (d <= 128 ? 4 : 8), dvb = dv <= 64 ? 4 : (dv <= 128 ? 8 : 16);
+    const int dk = d <= 64 ? 2 : (d <= 128 ? 4 : 8), dvb = dv <= 64 ? 4 : (dv <= 128 ? 8 : (dv <= 192 && d > 128 ? 12 : 16));
 #define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
   if (dk == DK && dvb == DVB)                                                                                                   \
     launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
                          ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, (hipStream_t)stream);
     NVS_MFMA_CASE(2, 4) NVS_MFMA_CASE(2, 8) NVS_MFMA_CASE(2, 16) NVS_MFMA_CASE(4, 4) NVS_MFMA_CASE(4, 8) NVS_MFMA_CASE(4, 16)
-    NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 16)
+    NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 12) NVS_MFMA_CASE(8, 16)
 #undef NVS_MFMA_CASE
     return nvs_check_launch("nvs_window_attn (matrix cores)");
   }

@@ -157,7 +157,7 @@ def run_mixer(m, w, h, second, dtype, block, cuts, path="auto", lend_to=None):
     mix.v_cache = torch.full(((pages + 3) * block, 1, m["kv_rank"]), -7.0, device="cuda", dtype=dtype)
     other = build_mixer(lend_to[0], lend_to[1], lend_to[2], dtype, block, source=mix, W=h.shape[1]) if lend_to else None
     assert other is None or other.kv_shapes() is None
-    ops_seq.load_library().nvs_window_attn_force_scalar({"auto": 0, "scalar": 1, "nolds": 2}[path])
+    ops_seq.load_library().nvs_window_attn_force_scalar({"auto": 0, "scalar": 1, "nolds": 2, "unpacked": 3}[path])
     outs, at = [], 0
     try:
         with torch.inference_mode():
@@ -184,13 +184,15 @@ def plain_mixer(m, w, h, second, kv=None):
 
 
 @pytest.mark.parametrize("dtype,path,tol", [(torch.float32, "auto", 3e-5), (torch.bfloat16, "auto", 3e-2), (torch.bfloat16, "nolds", 3e-2),
-                                            (torch.bfloat16, "scalar", 3e-2)])
+                                            (torch.bfloat16, "scalar", 3e-2), (torch.bfloat16, "unpacked", 3e-2)])
 @pytest.mark.parametrize("H,d,dr,dv,qr,r,window,second,rot,block", [
+    (8, 16, 8, 16, 24, 40, 23, False, ROTS[1], 16), (20, 8, 16, 24, 32, 176, 0, True, dict(ROTS[3], dims=16), 32), (70, 8, 8, 8, 16, 24, 50, False, ROTS[1], 64),
     (5, 24, 16, 40, 36, 48, 37, False, ROTS[0], 16), (4, 16, 32, 16, 24, 64, 0, True, ROTS[2], 64), (1, 8, 8, 8, 8, 16, 5, False, ROTS[1], 32),
     (3, 20, 12, 28, 50, 30, 0, True, ROTS[3], 16), (2, 64, 16, 64, 96, 200, 64, False, ROTS[0], 64), (2, 16, 16, 24, 20, 272, 70, False, ROTS[0], 16)])
 def test_latent_attention_against_the_plain_loop(H, d, dr, dv, qr, r, window, second, rot, block, dtype, path, tol):
     """One prompt portion, then short portions and single tokens; windows that do not line up with pages or query tiles, latent
-    rows that are not multiples of 8 or 16 and one longer than the matrix-core kernels take, one head, both pairings."""
+    rows that are not multiples of 8 or 16 and one longer than the matrix-core kernels take, one head, both pairings; with 8 heads
+    and more the single tokens run with heads packed into the query tiles (20: a partial tile; 70: two workgroups per token)."""
     T = 150
     m, w, h = latent_case(H, d, dr, dv, qr, r, window, second, rot, T, seed=H * 100 + r)
     want = plain_mixer(m, w, h, second)
