@@ -72,6 +72,8 @@ def load_library() -> ctypes.CDLL:
         lib.nvs_window_attn_force_scalar(1)
     elif os.environ.get("NVL_ATTN_NO_LDS") == "1":    # ... or on the matrix cores without the LDS-shared K / V tiles
         lib.nvs_window_attn_force_scalar(2)
+    elif os.environ.get("NVL_ATTN_UNPACKED") == "1":  # ... or never with heads in the query tiles of single-token steps
+        lib.nvs_window_attn_force_scalar(3)
     _lib = lib
     return lib
 
