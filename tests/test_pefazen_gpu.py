@@ -376,7 +376,7 @@ def small_config(variant: int = 0) -> dict:
                   dict(la(1, 8, 16, 8, 12, 32, 11, kv_from=0), mlp=moe(5, 1, 8)), dict(la(2, 12, 4, 20, 16, 20, 64), mlp=moe(2, 1, 32))]
         return {"architecture": "Pefazen", "vocab": 97, "width": 48, "layers": layers, "norm": {"eps": 1e-6}, "residual_mult": 1.0,
                 "logit_scale": 1.0, "logit_softcap": 30.0}
-    layers = [dict(la(4, 40, 32, 24, 64, 104, 130), mlp=moe(16, 4, 48)), dict(la2(10, 16, 8, 40, 56, 136), mlp=moe(8, 2, 96)),
+    layers = [dict(la(4, 40, 32, 24, 64, 104, 130), mlp=moe(16, 4, 48)), dict(la2(10, 16, 8, 40, 56, 144), mlp=moe(8, 2, 96)),
               dict(la(4, 24, 32, 16, 48, 104, 17, kv_from=0), mlp=moe(16, 2, 32))]
     return {"architecture": "Pefazen", "vocab": 384, "width": 256, "layers": layers, "norm": {"eps": 1e-5}, "residual_mult": 0.25,
             "logit_scale": 2.0}

@@ -320,3 +320,31 @@ def test_scaled_rotation_table_blends_between_the_two_marks():
     assert freq[0] == pytest.approx(plain[0]) and freq[1] == pytest.approx(plain[1] * (0.5 / 4 + 0.5))
     assert freq[2] == pytest.approx(plain[2] / 4) and freq[3] == pytest.approx(plain[3] / 4)
     assert rotary_frequencies(dims, base) == (plain, 1.0)
+
+
+def test_attention_in_the_latent_space_is_the_same_sum_reordered():
+    """What the product computes per head — scores of [W_uk^T q | rotated q part] against the cached row [c | rotated key part],
+    softmax, the weighted sum of the latents, then W_uv — equals the plain model's attention over up-projected keys and values
+    (float64, numpy; a window shorter than the sequence, gate included)."""
+    import numpy as np
+    from oracle import pefazen as plain
+    rng = np.random.default_rng(0)
+    n, W, H, d, dr, dv, qr, r, window = 23, 20, 3, 6, 4, 5, 7, 9, 8
+    m = {"heads": H, "dim": d, "rot_dim": dr, "vdim": dv, "q_rank": qr, "kv_rank": r, "scale": 0.4, "rot": {"dims": dr, "base": 50.0}, "mask": {"size": window}}
+    w = {"dq": rng.normal(size=(qr, W)), "dq.norm": rng.normal(size=qr), "uq": rng.normal(size=(H * (d + dr), qr)), "dkv": rng.normal(size=(r + dr, W)),
+         "dkv.norm": rng.normal(size=r), "uk": rng.normal(size=(H * d, r)), "uv": rng.normal(size=(H * dv, r)), "o": np.eye(H * dv), "g": rng.normal(size=(H, W))}
+    h = rng.normal(size=(n, W))
+    lat, kr = plain.latent_kv(h, w, m, 1e-5, False)
+    want = plain.latent_attention(h, w, m, 1e-5, False, window, True, (lat, kr))
+    freq, mag = plain.rotary_table(m["rot"])
+    q = (plain.rms_norm(h @ w["dq"].T, w["dq.norm"], 1e-5) @ w["uq"].T).reshape(n, H, d + dr)
+    rows = np.concatenate([lat, kr], 1)                                     # the cache: one row per token for all heads
+    got = np.zeros((n, H, dv))
+    for t in range(n):
+        keys = slice(max(t - window + 1, 0), t + 1)
+        for a in range(H):
+            qa = np.concatenate([w["uk"].reshape(H, d, r)[a].T @ q[t, a, :d], plain.rotate(q[t, a, d:], t, freq, mag, False)])
+            sc = rows[keys] @ qa * m["scale"]
+            p = np.exp(sc - sc.max())
+            got[t, a] = w["uv"].reshape(H, dv, r)[a] @ ((p / p.sum()) @ lat[keys]) / (1.0 + np.exp(-(h[t] @ w["g"][a])))
+    assert np.abs(got.reshape(n, H * dv) - want).max() < 1e-12
