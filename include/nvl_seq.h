@@ -48,6 +48,14 @@ int nvs_norm_residual(const void* m, const void* m2, const void* w1, const void*
 int nvs_add_group_norm(float* x, const void* a, float a_mult, const float* b, const int32_t* rows, int64_t nrows, const void* w,
                        int dtype, int width, int groups, float eps, int center, void* out, void* stream);
 
+/* Norms on both sides of a sublayer, on the 32-bit residual. The sublayer's output y[t, :] = a_mult * a[t, :] + a2_mult * a2[t, :]
+ * (a2 may be NULL) is divided by its root mean square and multiplied by (w_off + wa), and added: x[t, :] += rms(y) * (w_off + wa);
+ * then out[t, :] = rms(x[t, :]) * (w_off + w), the next sublayer's input. a == NULL: nothing is added; out == NULL: the add only.
+ * w_off = 1 serves weights that are stored as their distance from one. With rows != NULL nothing is added and out[r, :] is the
+ * norm of x[rows[r], :]. a, a2, wa, w, out in `dtype`; every sum in 32-bit. */
+int nvs_sandwich_norm(float* x, const void* a, float a_mult, const void* a2, float a2_mult, const void* wa, const int32_t* rows,
+                      int64_t nrows, const void* w, float w_off, int dtype, int width, float eps, void* out, void* stream);
+
 /* out[i] = cap * tanh(in[i] * scale / cap), or in[i] * scale with cap <= 0; in `dtype`, out 32-bit. */
 int nvs_scale_softcap(const void* in, int dtype, float scale, float cap, int64_t numel, float* out, void* stream);
 
@@ -62,10 +70,11 @@ int nvs_xielu(const void* in, const void* pq, float beta, int dtype, int64_t num
 /* Per-channel causal convolution over the packed portions, continuing each sequence from its state.
  * in: [n, channels] with row stride in_stride (elements, `dtype`); w [channels, taps] (last tap = current token), b [channels]
  * (nullable); act: 0 none, 1 SiLU. state [nslots, taps-1, channels] (32-bit) holds each sequence's last taps-1 inputs and
- * is advanced by the call (a second launch, after the outputs have been computed). out [n, channels], 32-bit. */
+ * is advanced by the call (a second launch, after the outputs have been computed). out [n, channels] in out_dtype: NVS_F32, or
+ * `dtype` itself (sums are 32-bit either way). */
 int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, const void* w, const void* b, int channels, int taps, int act,
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, const int32_t* tseq, int nseq, int64_t n,
-                    float* state, float* out, void* stream);
+                    float* state, void* out, int out_dtype, void* stream);
 
 /* Real-gated linear recurrence. gates [blocks, n, 2*bw] (32-bit): per block the pre-activations of the recurrence gate
  * (first bw) and of the input gate (last bw), biases included; u [n, C] 32-bit; ypre [n, C] (row stride y_stride) the
@@ -101,11 +110,25 @@ int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t
                    int heads, int dk, int dv, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
                    int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats, void* stream);
 
+/* The matrix memory with exponential gates, in 32-bit. Per head h and token, from the gate pre-activations zi, zf (columns i_col + h,
+ * f_col + h of proj [n, proj_stride], `dtype`, plus i_bias[h] / f_bias[h]): i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap));
+ * with the running maximum m (0 at a sequence's start): m' = max(f + m, i),
+ *   S <- exp(f + m - m') S + exp(i - m') k v^T,   n <- exp(f + m - m') n + exp(i - m') k,
+ * q (times q_scale), k (dk per head) and v (dv per head) being columns q_col / k_col / v_col (+ head * size) of proj, read as they
+ * are. y [n, heads * dv] receives the numerators S^T q, den [n, heads] the divisors max(|n . q|, exp(-m')) + 1e-6 (both 32-bit; the
+ * norm that follows divides: nvs_gated_group_norm's `den`). State: S [nslots, heads, dv + 1, dk] (row dv is n; dk fastest) and
+ * M [nslots, heads], advanced. The walk is nvs_ssd_scan's, one workgroup per (portion, head); never segmented. dv <= 256. */
+int nvs_gated_memory_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int64_t i_col, int64_t f_col,
+                          int dtype, const void* i_bias, const void* f_bias, float cap, float q_scale, int heads, int dk, int dv,
+                          const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n, float* S, float* M, float* y,
+                          float* den, void* stream);
+
 /* order 0: out = group_rms(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row by its own root mean
  * square. order 1: out = group_rms(y) * w * sigmoid(z): the norm first. y [n, inner] 32-bit; z [n, inner] with row stride z_stride
- * (`dtype`); w [inner]; out [n, inner] `dtype`. */
+ * (`dtype`); w [inner]; out [n, inner] `dtype`. den (nullable, order 1 only) [n, groups] 32-bit: every entry of group g of row t is
+ * divided by den[t, g] first. */
 int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
-                         float eps, int order, int64_t n, void* out, void* stream);
+                         float eps, int order, int64_t n, const float* den, void* out, void* stream);
 
 /* Key norm / rotation + paged K/V store. Rotation (rot_dims > 0, after the norm): entries (2i, 2i+1), i < rot_dims / 2, of every key head turn by
  * the angle pos[t] * rot_freq[i] (32-bit): (u, v) -> (u cos - v sin, v cos + u sin); the other entries pass. k [n, G, d] / v [n, G, dv] are column ranges of one projection output (row stride `stride`,
@@ -121,7 +144,9 @@ int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, c
  * q [n, H, d] (row stride q_stride), RMS-normed per head with qnorm [d] here (NULL: none), then rotated like the keys
  * (rot_dims, rot_freq; 0: not). Token t of portion s sits at position p = ctx0[s] + (t - cu_q[s]) and sees keys j with
  * 0 <= p - j < window (window > 0), or the keys j <= p of its own block, floor(j / chunk) == floor(p / chunk) (chunk > 0; blocks
- * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale, ordinary softmax in 32-bit. gate (nullable) [n, H*dv] with row stride
+ * are counted from position 0 of the sequence), or every j <= p (both 0), read through block_tables [nseq, bt_stride]. score = q.k * scale
+ * * (1 + qt_coef * ln(floor((p + 1) / qt_every) + 1)) (qt_every == 0: no such factor), softmax in 32-bit; with sink != NULL ([H],
+ * 32-bit) the denominator of head h also holds exp(sink[h]), a score that is not scaled and has no value. gate (nullable) [n, H*dv] with row stride
  * gate_stride: out *= sigmoid(gate); with gate_per_head != 0 the gate is [n, H], one entry for all columns of a head. out [n, H*dv] `dtype`.
  * bf16 with d % 8 == 0, d and dv <= 256 and block_size % 8 == 0 runs on the matrix cores (16 queries per wavefront — 16 positions of
  * one head, or in steps of single tokens with 8 or more query heads per kv head 16 heads at one position; the weights enter the
@@ -129,10 +154,12 @@ int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, int dtype, c
 int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_per_head, int dtype,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H, int G, int d, int dv,
-                    float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out, void* stream);
+                    float scale, int window, int chunk, const float* rot_freq, int rot_dims, const float* sink, float qt_coef, int qt_every,
+                    void* out, void* stream);
 
 /* Gated feed-forward activation on a fused [gate | up] projection: gu [n, 2 ff] with row stride `stride` -> out [n, ff] (`dtype`).
- * kind 0: silu(g) u. kind 1: g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' sigmoid(alpha g') (u' + 1). */
+ * kind 0: silu(g) u. kind 1: g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' sigmoid(alpha g') (u' + 1).
+ * kind 2: no gate at all, gu [n, ff]: out = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))). */
 int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, int kind, float limit, float alpha, int64_t n, void* out, void* stream);
 
 /* Routing of a mixture of experts, 32-bit. z [n, total] (row stride z_stride): router logits of all `total` entries.
@@ -142,6 +169,9 @@ int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, int kind, flo
  * the lower index. */
 int nvs_moe_route(const float* z, int64_t z_stride, const float* correction, int64_t n, int total, int top, int count, int keep, float scale,
                   int score, int renorm, int32_t* ids, float* wts, void* stream);
+
+/* Routing without a router: ids[t, k] = table[tokens[t], k] (table [vocab, top], int32; a row's entries differ), wts[t, k] = weight. */
+int nvs_moe_table_route(const int64_t* tokens, const int32_t* table, int64_t n, int top, float weight, int32_t* ids, float* wts, void* stream);
 
 /* Sort the pairs (token, choice) by expert. Pairs whose id >= experts have no rows (pass-through entries). Every expert's rows are
  * padded to whole tiles of tm (16, 64 or 128) rows; cap = nvs_moe_rows(n * top, experts, tm) rows are laid out.
@@ -161,7 +191,8 @@ int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype, int mode,
 void nvs_moe_force_plain(int on);
 
 /* out[t, :] = sum_k wts[t, k] * (pair_row[t, k] >= 0 ? rows[pair_row[t, k], :] : h[t, :]) + sigmoid(shared_gate[t]) * shared[t, :]
- * (shared NULL: no shared expert; shared_gate 32-bit pre-activations with row stride gate_stride). */
+ * (shared NULL: no shared expert; shared_gate 32-bit pre-activations with row stride gate_stride, NULL: the shared expert is added
+ * as it is). */
 int nvs_moe_combine(const void* rows, int64_t ldr, const int32_t* pair_row, const float* wts, int top, const void* h, int64_t ldh,
                     const void* shared, const float* shared_gate, int64_t gate_stride, int dtype, int64_t n, int width, void* out,
                     void* stream);

@@ -16,6 +16,12 @@ __device__ __forceinline__ int vis_lo(int p, int window, int chunk) {
   return 0;
 }
 
+// factor on the query at position p: 1 + coef * ln(floor((p + 1) / every) + 1) — a temperature that grows with the logarithm of the
+// position, in steps of `every` positions (every == 0: none)
+__device__ __forceinline__ float query_temp(int p, float coef, int every) {
+  return every > 0 ? 1.f + coef * logf((float)((p + 1) / every) + 1.f) : 1.f;
+}
+
 // one wavefront per (token, kv head)
 template <typename T, int CH>
 __global__ void knorm_kvstore_kernel(const T* __restrict__ k, const T* __restrict__ v, int64_t stride, const T* __restrict__ knorm,
@@ -67,7 +73,8 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
                                    const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int64_t bt_stride,
                                    int block_size, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ ctx0,
                                    const int32_t* __restrict__ tseq, int H, int G, int d, int dv, float scale, int window, int chunk,
-                                   const float* __restrict__ rot_freq, int rot_dims, T* __restrict__ out) {
+                                   const float* __restrict__ rot_freq, int rot_dims, const float* __restrict__ sink, float qt_coef,
+                                   int qt_every, T* __restrict__ out) {
   __shared__ float qs[CH * 64];
   __shared__ float ps[64];
   __shared__ int64_t slot_s[64];                    // element offset of (token, column 0) in the page-transposed V cache
@@ -104,7 +111,9 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
   __syncthreads();
   const int64_t lo = vis_lo((int)pos, window, chunk);
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
-  float m = -INFINITY, l = 0.f;
+  // a sink is a score in the denominator that has no value: the running maximum and sum start from it
+  float m = sink ? sink[h] : -INFINITY, l = sink ? 1.f : 0.f;
+  scale *= query_temp((int)pos, qt_coef, qt_every);
   float acc[CH];
 #pragma unroll
   for (int i = 0; i < CH; ++i) acc[i] = 0.f;
@@ -123,7 +132,7 @@ __global__ void window_attn_kernel(const T* __restrict__ q, int64_t q_stride, co
       sc = dot * scale;
     }
     const float mn = fmaxf(m, wave_max(sc));          // finite: lane 0 of every round is live
-    const float alpha = expf(m - mn);                 // 0 in the first round (m = -inf)
+    const float alpha = expf(m - mn);                 // 0 in the first round without a sink (m = -inf)
     const float p = live ? expf(sc - mn) : 0.f;
     l = l * alpha + wave_sum(p);
     m = mn;
@@ -181,7 +190,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
     int64_t gate_stride, int gate_w, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
-    const float* __restrict__ rot_freq, int rot_dims, int bs_shift, bf16_t* __restrict__ out) {
+    const float* __restrict__ rot_freq, int rot_dims, const float* __restrict__ sink, float qt_coef, int qt_every,
+    int bs_shift, bf16_t* __restrict__ out) {
   constexpr int QW = 16 * QT;                       // queries per wavefront
   const int lane = threadIdx.x & 63, qi = lane & 15, gq = lane >> 4;
   int tile = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -222,7 +232,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
         qv[c][e] = col < d ? (float)qp[col] : 0.f;
         ss += qv[c][e] * qv[c][e];
       }
-    float r = scale;
+    float r = scale * query_temp(pos[t], qt_coef, qt_every);
     if (qnorm) {
       ss += __shfl_xor(ss, 16, 64);
       ss += __shfl_xor(ss, 32, 64);
@@ -254,8 +264,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
   f32x4_t oacc[QT][DVB];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    m[t] = -1e30f;
-    lsum[t] = 0.f;
+    m[t] = sink ? sink[h] : -1e30f;                 // a sink: a score in the denominator without a value (counted once: by gq 0)
+    lsum[t] = sink && gq == 0 ? 1.f : 0.f;
 #pragma unroll
     for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -384,7 +394,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
     int64_t gate_stride, int gate_w, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int64_t bt_stride, int block_size, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ ctx0, int nseq, int H, int G, int d, int dv, float scale, int window, int chunk,
-    const float* __restrict__ rot_freq, int rot_dims, int bs_shift, int hw, bf16_t* __restrict__ out) {
+    const float* __restrict__ rot_freq, int rot_dims, const float* __restrict__ sink, float qt_coef, int qt_every,
+    int bs_shift, int hw, bf16_t* __restrict__ out) {
   constexpr int QW = 16 * QT, KP = 32 * DK + 8, VP = 64 + 8, VU = DVB / 2;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[64][KP];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * DVB][VP];
@@ -437,7 +448,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
         qv[c][e] = col < d ? (float)qp[col] : 0.f;
         ss += qv[c][e] * qv[c][e];
       }
-    float r = scale;
+    float r = scale * query_temp(pos[t], qt_coef, qt_every);
     if (qnorm) {
       ss += __shfl_xor(ss, 16, 64);
       ss += __shfl_xor(ss, 32, 64);
@@ -466,8 +477,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
   f32x4_t oacc[QT][DVB];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    m[t] = -1e30f;
-    lsum[t] = 0.f;
+    m[t] = sink ? sink[hq[t]] : -1e30f;             // a sink: a score in the denominator without a value (counted once: by gq 0)
+    lsum[t] = sink && gq == 0 ? 1.f : 0.f;
 #pragma unroll
     for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -622,7 +633,7 @@ template <int DK, int DVB, int QT>
 void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_w,
                     const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                     const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
-                    int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
+                    int chunk, const float* rot_freq, int rot_dims, const float* sink, float qt_coef, int qt_every, void* out, hipStream_t stream) {
   int bs_shift = -1;
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == block_size) bs_shift = b;
@@ -635,7 +646,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
           window_attn_mfma_lds_kernel<DK, DVB, 1><<<dim3((unsigned)n, (unsigned)(G * ((hpg + 63) / 64))), dim3(256), 0, stream>>>(
               (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
               (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq,
-              rot_dims, bs_shift, 0, (bf16_t*)out);
+              rot_dims, sink, qt_coef, qt_every, bs_shift, 0, (bf16_t*)out);
           return;
         }
       }
@@ -645,7 +656,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
       window_attn_mfma_lds_kernel<DK, DVB, QT><<<dim3((unsigned)btiles, (unsigned)(G * (hpg / hw))), dim3(256), 0, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
           (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq,
-          rot_dims, bs_shift, hw, (bf16_t*)out);
+          rot_dims, sink, qt_coef, qt_every, bs_shift, hw, (bf16_t*)out);
       return;
     }
   }
@@ -653,7 +664,7 @@ void launch_mfma_qt(const void* q, int64_t q_stride, const void* qnorm, float ep
   window_attn_mfma_kernel<DK, DVB, QT><<<dim3((unsigned)((tiles + 3) / 4), H), dim3(256), 0, stream>>>(
       (const bf16_t*)q, q_stride, (const bf16_t*)qnorm, eps, (const bf16_t*)gate, gate_stride, gate_w, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, nseq, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims,
-      bs_shift, (bf16_t*)out);
+      sink, qt_coef, qt_every, bs_shift, (bf16_t*)out);
 }
 
 // Long portions (prefill) put two tiles of 16 queries on a wavefront: half the K / V bytes through the vector cache per
@@ -662,13 +673,13 @@ template <int DK, int DVB>
 void launch_mfma(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride, int gate_w,
                  const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride, int block_size,
                  const int32_t* cu_q, const int32_t* ctx0, int nseq, int64_t n, int H, int G, int d, int dv, float scale, int window,
-                 int chunk, const float* rot_freq, int rot_dims, void* out, hipStream_t stream) {
+                 int chunk, const float* rot_freq, int rot_dims, const float* sink, float qt_coef, int qt_every, void* out, hipStream_t stream) {
   if (n >= 32ll * nseq)
     launch_mfma_qt<DK, DVB, 2>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
-                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
+                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, sink, qt_coef, qt_every, out, stream);
   else
     launch_mfma_qt<DK, DVB, 1>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q,
-                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, stream);
+                               ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, sink, qt_coef, qt_every, out, stream);
 }
 }  // namespace
 
@@ -703,8 +714,9 @@ extern "C" int nvs_knorm_kvstore(const void* k, const void* v, int64_t stride, i
 extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnorm, float eps, const void* gate, int64_t gate_stride,
                                int gate_per_head, int dtype, const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride,
                                int block_size, const int32_t* cu_q, const int32_t* ctx0, const int32_t* tseq, int nseq, int64_t n, int H,
-                               int G, int d, int dv, float scale, int window, int chunk, const float* rot_freq, int rot_dims, void* out,
-                               void* stream) {
+                               int G, int d, int dv, float scale, int window, int chunk, const float* rot_freq, int rot_dims, const float* sink,
+                               float qt_coef, int qt_every, void* out, void* stream) {
+  NVS_REQUIRE(qt_every >= 0, "nvs_window_attn: a query temperature every %d positions", qt_every);
   NVS_REQUIRE(q && k_cache && v_cache && block_tables && cu_q && ctx0 && tseq && out, "nvs_window_attn: null argument");
   NVS_REQUIRE(!(window > 0 && chunk > 0), "nvs_window_attn: a window (%d) and blocks (%d) together", window, chunk);
   NVS_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= d && (rot_dims == 0 || rot_freq),
@@ -718,7 +730,7 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
 #define NVS_MFMA_CASE(DK, DVB)                                                                                                  \
   if (dk == DK && dvb == DVB)                                                                                                   \
     launch_mfma<DK, DVB>(q, q_stride, qnorm, eps, gate, gate_stride, gate_w, k_cache, v_cache, block_tables, bt_stride, block_size, cu_q, \
-                         ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, out, (hipStream_t)stream);
+                         ctx0, nseq, n, H, G, d, dv, scale, window, chunk, rot_freq, rot_dims, sink, qt_coef, qt_every, out, (hipStream_t)stream);
     NVS_MFMA_CASE(2, 4) NVS_MFMA_CASE(2, 8) NVS_MFMA_CASE(2, 16) NVS_MFMA_CASE(4, 4) NVS_MFMA_CASE(4, 8) NVS_MFMA_CASE(4, 16)
     NVS_MFMA_CASE(8, 4) NVS_MFMA_CASE(8, 8) NVS_MFMA_CASE(8, 12) NVS_MFMA_CASE(8, 16)
 #undef NVS_MFMA_CASE
@@ -728,11 +740,11 @@ extern "C" int nvs_window_attn(const void* q, int64_t q_stride, const void* qnor
     NVS_DISPATCH(dtype, window_attn_kernel<T, 4><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
                             (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache,
                             (const T*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq,
-                            rot_dims, (T*)out));
+                            rot_dims, sink, qt_coef, qt_every, (T*)out));
   else                                               // heads of up to 1024 entries: the same kernel with 16 entries per lane
     NVS_DISPATCH(dtype, window_attn_kernel<T, 16><<<dim3((unsigned)n, H), dim3(64), 0, (hipStream_t)stream>>>(
                             (const T*)q, q_stride, (const T*)qnorm, eps, (const T*)gate, gate_stride, gate_w, (const T*)k_cache,
                             (const T*)v_cache, block_tables, bt_stride, block_size, cu_q, ctx0, tseq, H, G, d, dv, scale, window, chunk, rot_freq,
-                            rot_dims, (T*)out));
+                            rot_dims, sink, qt_coef, qt_every, (T*)out));
   return nvs_check_launch("nvs_window_attn");
 }

@@ -18,6 +18,7 @@ constexpr int MAX_EXPERTS = 1024;
 
 __device__ __forceinline__ float glu_value(float g, float u, int kind, float limit, float alpha) {
   if (kind == 0) return g / (1.f + expf(-g)) * u;               // silu(g) * u
+  if (kind == 2) return gelu_tanhf_(g);                         // ungated: the tanh form of GELU (u is not read)
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);              // clamped: g sigmoid(alpha g) (u + 1)
@@ -37,8 +38,18 @@ __global__ void glu_act_kernel(const T* __restrict__ gu, int64_t stride, int ff,
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / ff;
     const int c = (int)(i - t * ff);
-    stf(out + i, glu_value(ldf(gu + t * stride + c), ldf(gu + t * stride + ff + c), kind, limit, alpha));
+    stf(out + i, glu_value(ldf(gu + t * stride + c), kind == 2 ? 0.f : ldf(gu + t * stride + ff + c), kind, limit, alpha));
   }
+}
+
+// ---- routing without a router: a table row per token id names the token's experts, all with the same weight ----------
+__global__ void moe_table_route_kernel(const int64_t* __restrict__ tokens, const int32_t* __restrict__ table, int64_t pairs, int top,
+                                       float weight, int32_t* __restrict__ ids, float* __restrict__ wts) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= pairs) return;
+  const int64_t t = i / top;
+  ids[i] = table[tokens[t] * top + (i - t * top)];
+  wts[i] = weight;
 }
 
 // ---- routing: one wavefront per token, a lane holds entries lane, lane + 64, ... of the token's scores ---------------
@@ -404,7 +415,7 @@ __global__ void moe_combine_kernel(const T* __restrict__ rows, int64_t ldr, cons
                                    T* __restrict__ out) {
   const int64_t t = blockIdx.x;
   float sg = 0.f;
-  if (shared) sg = 1.f / (1.f + expf(-shared_gate[t * gate_stride]));
+  if (shared) sg = shared_gate ? 1.f / (1.f + expf(-shared_gate[t * gate_stride])) : 1.f;      // no gate: the shared expert is added as it is
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
@@ -424,7 +435,7 @@ extern "C" void nvs_moe_force_plain(int on) { g_moe_plain = on; }
 
 extern "C" int nvs_glu_act(const void* gu, int64_t stride, int dtype, int ff, int kind, float limit, float alpha, int64_t n, void* out,
                            void* stream) {
-  NVS_REQUIRE(gu && out && ff > 0 && stride >= 2 * (int64_t)ff && (kind == 0 || kind == 1) && n >= 0, "nvs_glu_act: ff %d stride %lld kind %d",
+  NVS_REQUIRE(gu && out && ff > 0 && stride >= (kind == 2 ? 1 : 2) * (int64_t)ff && kind >= 0 && kind <= 2 && n >= 0, "nvs_glu_act: ff %d stride %lld kind %d",
               ff, (long long)stride, kind);
   if (n == 0) return NVS_OK;
   int64_t blocks = (n * ff + 255) / 256;
@@ -443,6 +454,15 @@ extern "C" int nvs_moe_route(const float* z, int64_t z_stride, const float* corr
   if (n == 0) return NVS_OK;
   moe_route_kernel<<<dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream>>>(z, z_stride, correction, total, top, count, keep, scale, score, renorm, ids, wts);
   return nvs_check_launch("nvs_moe_route");
+}
+
+extern "C" int nvs_moe_table_route(const int64_t* tokens, const int32_t* table, int64_t n, int top, float weight, int32_t* ids, float* wts,
+                                   void* stream) {
+  NVS_REQUIRE(tokens && table && ids && wts && n >= 0 && top > 0 && top <= 64, "nvs_moe_table_route: bad argument (%d choices)", top);
+  if (n == 0) return NVS_OK;
+  const int64_t pairs = n * top;
+  moe_table_route_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(tokens, table, pairs, top, weight, ids, wts);
+  return nvs_check_launch("nvs_moe_table_route");
 }
 
 extern "C" int64_t nvs_moe_rows(int64_t pairs, int experts, int tm) { return (pairs + (int64_t)experts * (tm - 1) + tm - 1) / tm * tm; }
@@ -507,7 +527,7 @@ extern "C" int nvs_moe_gemm(const void* X, int64_t ldx, const void* W, int dtype
 extern "C" int nvs_moe_combine(const void* rows, int64_t ldr, const int32_t* pair_row, const float* wts, int top, const void* h, int64_t ldh,
                                const void* shared, const float* shared_gate, int64_t gate_stride, int dtype, int64_t n, int width, void* out,
                                void* stream) {
-  NVS_REQUIRE(rows && pair_row && wts && h && out && top > 0 && width > 0 && n >= 0 && (!shared || shared_gate),
+  NVS_REQUIRE(rows && pair_row && wts && h && out && top > 0 && width > 0 && n >= 0,
               "nvs_moe_combine: bad argument");
   if (n == 0) return NVS_OK;
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);

@@ -20,7 +20,7 @@ int nvs_check_launch(const char* what) {
   }
   return NVS_OK;
 }
-extern "C" int nvs_abi_version(void) { return 4; }   // 4: centered norms and scaled adds, latent attention, sigmoid routers, logit cap
+extern "C" int nvs_abi_version(void) { return 5; }   // 5: norms on both sides of a sublayer, attention sinks and query temperature, the gated matrix memory, table-routed experts
 extern "C" const char* nvs_last_error(void) { return g_err; }
 
 namespace {
@@ -169,6 +169,42 @@ __global__ void add_group_norm_kernel(float* __restrict__ x, const T* __restrict
   }
 }
 
+// Norms on BOTH sides of a sublayer, on the 32-bit residual: the sublayer's output y[t] = a_mult * a[t] + a2_mult * a2[t] (a2 may be
+// absent) is RMS-normed with the weight (w_off + wa) and added, x[t] += rms(y[t]) * (w_off + wa); then the NEXT sublayer's input
+// out[t] = rms(x[t]) * (w_off + w). Either half may be absent (a NULL / out NULL). w_off = 1 serves weights stored as their distance
+// from one. With `rows` the kernel only reads: out[r] = norm(x[rows[r]]). One workgroup per row; all sums in 32-bit.
+template <typename T>
+__global__ void sandwich_norm_kernel(float* __restrict__ x, const T* __restrict__ a, float a_mult, const T* __restrict__ a2, float a2_mult,
+                                     const T* __restrict__ wa, const int32_t* __restrict__ rows, const T* __restrict__ w, float w_off,
+                                     int width, float eps, T* __restrict__ out) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t t = rows ? (int64_t)rows[r] : r;
+  float* xr = x + t * width;
+  if (a) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      float y = a_mult * ldf(a + t * width + c);
+      if (a2) y += a2_mult * ldf(a2 + t * width + c);
+      ss += y * y;
+    }
+    const float k = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      float y = a_mult * ldf(a + t * width + c);
+      if (a2) y += a2_mult * ldf(a2 + t * width + c);
+      xr[c] += y * k * (w_off + ldf(wa + c));
+    }
+  }
+  if (!out) return;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {     // (every thread reads back what it wrote itself)
+    const float v = xr[c];
+    ss += v * v;
+  }
+  const float k = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) stf(out + r * width + c, xr[c] * k * (w_off + ldf(w + c)));
+}
+
 // logits <- cap * tanh(logits * scale / cap) (cap <= 0: logits * scale), 32-bit out
 template <typename T>
 __global__ void scale_softcap_kernel(const T* __restrict__ in, float scale, float cap, int64_t numel, float* __restrict__ out) {
@@ -231,6 +267,16 @@ extern "C" int nvs_add_group_norm(float* x, const void* a, float a_mult, const f
   NVS_DISPATCH(dtype, add_group_norm_kernel<T><<<dim3((unsigned)nrows), dim3(threads), 0, (hipStream_t)stream>>>(
                           x, (const T*)a, a_mult, b, rows, (const T*)w, width, groups, eps, center, (T*)out));
   return nvs_check_launch("nvs_add_group_norm");
+}
+
+extern "C" int nvs_sandwich_norm(float* x, const void* a, float a_mult, const void* a2, float a2_mult, const void* wa, const int32_t* rows,
+                                 int64_t nrows, const void* w, float w_off, int dtype, int width, float eps, void* out, void* stream) {
+  NVS_REQUIRE(x && nrows >= 0 && width > 0 && (a || out) && (!a || wa) && (!a2 || a) && (!out || w), "nvs_sandwich_norm: bad argument (width %d)", width);
+  NVS_REQUIRE(!rows || !a, "nvs_sandwich_norm: selected rows are only read");
+  if (nrows == 0) return NVS_OK;
+  NVS_DISPATCH(dtype, sandwich_norm_kernel<T><<<dim3((unsigned)nrows), dim3(threads_for(width)), 0, (hipStream_t)stream>>>(
+                          x, (const T*)a, a_mult, (const T*)a2, a2_mult, (const T*)wa, rows, (const T*)w, w_off, width, eps, (T*)out));
+  return nvs_check_launch("nvs_sandwich_norm");
 }
 
 extern "C" int nvs_scale_softcap(const void* in, int dtype, float scale, float cap, int64_t numel, float* out, void* stream) {

@@ -10,11 +10,11 @@ constexpr int MAX_TAPS = 8;
 
 // ---- causal convolution -------------------------------------------------------------------------------------------
 // one thread per (token, channel); inputs before the portion come from the slot's tail (or are zero at a sequence start)
-template <typename T>
+template <typename T, typename TO>
 __global__ void causal_conv_kernel(const T* __restrict__ in, int64_t in_stride, const T* __restrict__ w, const T* __restrict__ b,
                                    int channels, int taps, int act, const int32_t* __restrict__ cu_q,
                                    const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot,
-                                   const int32_t* __restrict__ tseq, const float* __restrict__ state, float* __restrict__ out,
+                                   const int32_t* __restrict__ tseq, const float* __restrict__ state, TO* __restrict__ out,
                                    int64_t t0) {
   const int64_t t = t0 + blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -40,7 +40,7 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, int64_t in_stride, 
     acc += ldf(w + (int64_t)c * taps + j) * v;
   }
   if (act == 1) acc = siluf_(acc);
-  out[t * channels + c] = acc;
+  stf(out + t * channels + c, acc);
 }
 
 // one thread per (portion, channel): the new tail is read completely before it is written
@@ -165,13 +165,23 @@ constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken togethe
 // ("lightning") attention, S <- decay_h S + k v^T, o = S^T q — the same walk with x = v, B = k, C = q, a step size of one, a
 // decay that is a per-head constant (`decay`, 32-bit) and no skip term; v | k | q are read from the projection output itself
 // (columns x_col / b_col / c_col + the head's offset, `dtype`) and SiLU is applied as they are staged.
+// FORM 2: the matrix memory with exponential gates. Per head and token, from the gate pre-activations zi, zf (columns i_col / f_col
+// + head of the projection output, plus a bias each): i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)); with a running
+// maximum m (0 at a sequence's start) m' = max(f + m, i), S <- exp(f + m - m') S + exp(i - m') k v^T, n likewise with k alone. The
+// walk is the same with x = v, B = k, C = q * c_scale, decay exp(f + m - m'), step exp(i - m') — ONE thread turns the round's gates
+// into these, token after token, while the others stage the operands — and n is simply one more row of the state, whose "value" is
+// the constant 1: the kernel sees P = dv + 1 rows (state memory [heads][dv + 1][dk], M [nslots][heads] holds m). It writes the
+// numerators S^T q to y [n, heads * dv] and den [n, heads] = max(|n . q|, exp(-m')) + 1e-6; the division is left to the norm that
+// follows. Never segmented (a segment's maximum depends on all tokens before it).
 template <typename T, int PP, int MODE, int FORM = 0>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
-__global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+__global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)) : (PP == 4 ? 256 : (PP == 2 ? 512 : 1024))) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 int64_t x_col, int64_t b_col, int64_t c_col, const float* __restrict__ decay,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
                                 const int32_t* __restrict__ ctx0, const int32_t* __restrict__ slot, float* __restrict__ S,
-                                float* __restrict__ y, int seg_len, int nseg, float* __restrict__ ws) {
+                                float* __restrict__ y, int seg_len, int nseg, float* __restrict__ ws, int64_t i_col, int64_t f_col,
+                                const T* __restrict__ i_bias, const T* __restrict__ f_bias, float cap, float c_scale,
+                                float* __restrict__ M, float* __restrict__ den) {
   constexpr int mode = MODE;                        // (compile-time: the unsegmented scan pays nothing for the other two)
   // mode 0: the whole portion in one workgroup. Long portions with few (portion, head) pairs are cut into segments of
   // seg_len tokens (blockIdx.z) and scanned twice, because one workgroup walks its tokens one after the other:
@@ -202,6 +212,13 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   float* Sh = S + (((int64_t)slot[s] * heads + h) * P + p) * N + g * SSD_R;
   float st[PP][SSD_R];
   const bool fresh = ctx0[s] == 0;
+  // FORM 2: the running maximum (kept by the one thread that turns gates into decays), the gates' biases, rows beyond P are idle
+  const int Py = FORM == 2 ? P - 1 : P;             // rows that are outputs
+  float mrun = 0.f, bi = 0.f, bf = 0.f;
+  if (FORM == 2) {
+    bi = ldf(i_bias + h), bf = ldf(f_bias + h);
+    if (!fresh) mrun = M[(int64_t)slot[s] * heads + h];
+  }
   const bool vec = (N & 3) == 0;                    // a thread's 16 entries are then four aligned 16-byte pieces
   auto load16 = [&](const float* src, float (&dst)[SSD_R]) {
     if (vec) {
@@ -240,7 +257,7 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
 #pragma unroll
         for (int r = 0; r < SSD_R; ++r) st[i][r] = dk * st[i][r] + lk[r];
       }
-    } else if (!fresh && (mode == 0 || seg == 0)) {
+    } else if (!fresh && (mode == 0 || seg == 0) && (FORM != 2 || p + i < P)) {
       load16(Sh + (int64_t)i * N, st[i]);
     }
     if (mode == 1 && seg == 0) {                    // the portion's starting state, for mode 2
@@ -253,10 +270,11 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
   float dprod = 1.f;
 
   const float* xh = xbc + h * P;
-  float* yh = y + h * P + p;
+  float* yh = y + h * Py + p;
+  const int inner_y = heads * Py;
   const float* Bg = xbc + inner + grp * N;
   const float* Cg = Bg + G * N;
-  const T* xh1 = proj + x_col + h * P;              // FORM 1: the three operands inside the projection output
+  const T* xh1 = proj + x_col + h * Py;             // FORM 1, 2: the three operands inside the projection output
   const T* Bg1 = proj + b_col + grp * N;
   const T* Cg1 = proj + c_col + grp * N;
   for (int64_t tb = q0; tb < q1; tb += TB) {
@@ -269,18 +287,47 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
       const float* src = nullptr;                   // a 32-bit source with row stride `row`
       const T* src1 = nullptr;                      // FORM 1: a source in the projection output, SiLU applied here
       int kind = 0;                                 // 0: padding (zero), 1: x / B / C, 2: step size, 3: decay
-      if (c < P) {
+      if (FORM == 2 && c == P - 1) {
+        kind = 4;                                   // the normaliser's row: its "value" is the constant 1
+      } else if (c < P) {
         src = xh + c, src1 = xh1 + c, kind = 1;
       } else if (c >= P4 && c < P4 + NP) {
         if (c - P4 < N) src = Bg + (c - P4), src1 = Bg1 + (c - P4), kind = 1;
       } else if (c >= P4 + NP && c < P4 + 2 * NP) {
-        if (c - P4 - NP < N) src = Cg + (c - P4 - NP), src1 = Cg1 + (c - P4 - NP), kind = 1;
+        if (c - P4 - NP < N) src = Cg + (c - P4 - NP), src1 = Cg1 + (c - P4 - NP), kind = FORM == 2 ? 5 : 1;
       } else if (c == P4 + 2 * NP) {
         kind = 2;
       } else if (c == P4 + 2 * NP + 1) {
         kind = 3;
       }
       float v[SSD_TB];
+      if (FORM == 2 && kind == 2) {
+        // this thread alone: the round's gates -> step, decay and exp(-m) of every token, in order (m runs through the portion)
+        float zi[SSD_TB], zf[SSD_TB];
+#pragma unroll
+        for (int k = 0; k < SSD_TB; ++k) {
+          zi[k] = zf[k] = 0.f;
+          if (k < cnt) {
+            zi[k] = ldf(proj + (tb + k) * proj_stride + i_col + h);
+            zf[k] = ldf(proj + (tb + k) * proj_stride + f_col + h);
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < SSD_TB; ++k) {
+          if (k < cnt) {
+            const float gi = cap * tanhf((zi[k] + bi) / cap);
+            const float zc = cap * tanhf((zf[k] + bf) / cap);
+            const float gf = fminf(zc, 0.f) - log1pf(expf(-fabsf(zc)));          // log sigmoid
+            const float mn = fmaxf(gf + mrun, gi);
+            lds[k * per + c] = expf(gi - mn);
+            lds[k * per + c + 1] = expf(gf + mrun - mn);
+            lds[k * per + c + 2] = expf(-mn);
+            mrun = mn;
+          }
+        }
+        continue;
+      }
+      if (FORM == 2 && c > P4 + 2 * NP) continue;   // (decay, exp(-m) and the spare entry belong to the thread beside)
 #pragma unroll
       for (int k = 0; k < SSD_TB; ++k) {
         v[k] = 0.f;
@@ -289,7 +336,7 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
             if (kind == 1) v[k] = src[(tb + k) * row];
             if (kind >= 2) v[k] = ldf(proj + (tb + k) * proj_stride + dt_col + h);
           } else {
-            if (kind == 1) v[k] = ldf(src1 + (tb + k) * proj_stride);
+            if (kind == 1 || kind == 5) v[k] = ldf(src1 + (tb + k) * proj_stride);
           }
         }
       }
@@ -302,10 +349,13 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
               w = softplusf_(w + dtb);
               if (kind == 3) w = expf(A * w);
             }
-          } else {
+          } else if (FORM == 1) {
             if (kind == 1) w = siluf_(w);
             if (kind == 2) w = 1.f;
             if (kind == 3) w = fixed_decay;
+          } else {
+            if (kind == 4) w = 1.f;
+            if (kind == 5) w *= c_scale;
           }
           lds[k * per + c] = w;
         }
@@ -324,7 +374,7 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
       for (int r = 0; r < SSD_R; ++r) bv[r] = Bp[r], cv[r] = Cp[r];
 #pragma unroll
       for (int i = 0; i < PP; ++i) {
-        const float xv = tp[p + i];
+        const float xv = (FORM != 2 || p + i < P) ? tp[p + i] : 0.f;
         const float dx = dt * xv;
         float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
@@ -359,7 +409,14 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
 #pragma unroll
           for (int k = 0; k < SSD_SB; ++k)
 #pragma unroll
-            for (int i = 0; i < PP; ++i) yh[(tb + k0 + k) * inner + i] = part[k][i] + Dh * xs[k][i];
+            for (int i = 0; i < PP; ++i) {
+              if (FORM == 2) {
+                if (p + i < Py) yh[(tb + k0 + k) * inner_y + i] = part[k][i];
+                else if (p + i == Py) den[(tb + k0 + k) * heads + h] = fmaxf(fabsf(part[k][i]), lds[(k0 + k) * per + P4 + 2 * NP + 2]) + 1e-6f;
+              } else {
+                yh[(tb + k0 + k) * inner + i] = part[k][i] + Dh * xs[k][i];
+              }
+            }
         }
       }
     } else {
@@ -370,7 +427,14 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
         for (int i = 0; i < PP; ++i) {
           float acc = part[i];
           for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-          if (g == 0 && mode != 1) yh[(tb + k) * inner + i] = acc + Dh * xs[i];
+          if (g == 0 && mode != 1) {
+            if (FORM == 2) {
+              if (p + i < Py) yh[(tb + k) * inner_y + i] = acc;
+              else if (p + i == Py) den[(tb + k) * heads + h] = fmaxf(fabsf(acc), lds[k * per + P4 + 2 * NP + 2]) + 1e-6f;
+            } else {
+              yh[(tb + k) * inner + i] = acc + Dh * xs[i];
+            }
+          }
         }
       }
     }
@@ -381,7 +445,9 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
     if (tid == 0) wdec[seg + 1] = dprod;
   } else if (last) {
 #pragma unroll
-    for (int i = 0; i < PP; ++i) store16(Sh + (int64_t)i * N, st[i]);
+    for (int i = 0; i < PP; ++i)
+      if (FORM != 2 || p + i < P) store16(Sh + (int64_t)i * N, st[i]);
+    if (FORM == 2 && tid == (P4 + 2 * NP) % nthreads) M[(int64_t)slot[s] * heads + h] = mrun;      // the thread that kept it
   }
 }
 
@@ -389,20 +455,22 @@ __global__ __launch_bounds__(PP == 4 ? 256 : (PP == 2 ? 512 : 1024)) void ssd_sc
 // one workgroup per (token, group)
 template <typename T>
 __global__ void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int64_t z_stride,
-                                        const T* __restrict__ w, int inner, int groups, float eps, int order, T* __restrict__ out) {
+                                        const T* __restrict__ w, int inner, int groups, float eps, int order,
+                                        const float* __restrict__ den, T* __restrict__ out) {
   __shared__ float red[16];
   const int64_t t = blockIdx.y;
   const int gsz = inner / groups, c0 = blockIdx.x * gsz;
   float ss = 0.f;
   if (order == 1) {                                 // norm first, then a sigmoid gate
+    const float dinv = den ? 1.f / den[t * groups + blockIdx.x] : 1.f;      // the group's entries are numerators over this
     for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
-      const float v = y[t * inner + c0 + c];
+      const float v = y[t * inner + c0 + c] * dinv;
       ss += v * v;
     }
     const float r = 1.f / sqrtf(block_sum(ss, red) / (float)gsz + eps);
     for (int c = threadIdx.x; c < gsz; c += blockDim.x) {
       const float gz = ldf(z + t * z_stride + c0 + c);
-      stf(out + t * inner + c0 + c, y[t * inner + c0 + c] * r * ldf(w + c0 + c) * (1.f / (1.f + expf(-gz))));
+      stf(out + t * inner + c0 + c, y[t * inner + c0 + c] * dinv * r * ldf(w + c0 + c) * (1.f / (1.f + expf(-gz))));
     }
     return;
   }
@@ -421,7 +489,8 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ y, const T* __
 
 extern "C" int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, const void* w, const void* b, int channels, int taps,
                                int act, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, const int32_t* tseq, int nseq,
-                               int64_t n, float* state, float* out, void* stream) {
+                               int64_t n, float* state, void* out, int out_dtype, void* stream) {
+  NVS_REQUIRE(out_dtype == NVS_F32 || out_dtype == dtype, "nvs_causal_conv: the output is 32-bit or of the input's type");
   NVS_REQUIRE(in && w && cu_q && ctx0 && slot && tseq && (state || taps == 1) && out, "nvs_causal_conv: null argument");
   NVS_REQUIRE(channels > 0 && taps >= 1 && taps <= MAX_TAPS && in_stride >= channels && nseq >= 0 && n >= 0 && (act == 0 || act == 1),
               "nvs_causal_conv: channels %d taps %d (1..%d) stride %lld act %d", channels, taps, MAX_TAPS, (long long)in_stride, act);
@@ -432,9 +501,14 @@ extern "C" int nvs_causal_conv(const void* in, int64_t in_stride, int dtype, con
   // grid.y is limited to 65535: larger steps go in slices
   for (int64_t t0 = 0; t0 < n; t0 += 65535) {
     const int64_t cnt = n - t0 < 65535 ? n - t0 : 65535;
-    NVS_DISPATCH(dtype, causal_conv_kernel<T><<<dim3(gx, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
-                            (const T*)in, in_stride, (const T*)w, (const T*)b, channels, taps, act, cu_q, ctx0, slot, tseq, state, out,
-                            t0));
+    if (out_dtype == NVS_F32)
+      NVS_DISPATCH(dtype, causal_conv_kernel<T, float><<<dim3(gx, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
+                              (const T*)in, in_stride, (const T*)w, (const T*)b, channels, taps, act, cu_q, ctx0, slot, tseq, state,
+                              (float*)out, t0));
+    else
+      NVS_DISPATCH(dtype, causal_conv_kernel<T, T><<<dim3(gx, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
+                              (const T*)in, in_stride, (const T*)w, (const T*)b, channels, taps, act, cu_q, ctx0, slot, tseq, state,
+                              (T*)out, t0));
   }
   int rc = nvs_check_launch("nvs_causal_conv");
   if (rc) return rc;
@@ -496,12 +570,20 @@ extern "C" int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int
   return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)P * N + 1) : 0;
 }
 
-// both forms of the scan: argument checks that they share, the plan, the launches
+// what only the matrix memory (form 2) passes
+struct GateArgs {
+  int64_t i_col = 0, f_col = 0;
+  const void *i_bias = nullptr, *f_bias = nullptr;
+  float cap = 0.f, c_scale = 1.f;
+  float *M = nullptr, *den = nullptr;
+};
+
+// all forms of the scan: argument checks that they share, the plan, the launches
 static int ssd_launch(int form, const char* who, const float* xbc, const void* proj, int64_t proj_stride, int64_t dt_col, int64_t x_col,
                       int64_t b_col, int64_t c_col, const float* decay, int dtype, const void* dt_bias, const void* A_log, const void* D,
                       int heads, int P, int N, int G, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
-                      int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats, void* stream) {
-  NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 256 && N > 0 && nseq >= 0 && nseq <= 65535,
+                      int64_t max_q, float* S, float* y, float* ws, int64_t ws_floats, void* stream, const GateArgs& ga = GateArgs()) {
+  NVS_REQUIRE(heads > 0 && G > 0 && heads % G == 0 && P > 0 && P <= 257 && N > 0 && nseq >= 0 && nseq <= 65535,
               "%s: heads %d groups %d head size %d state %d", who, heads, G, P, N);
   if (n == 0 || nseq == 0) return NVS_OK;
   int ng = 1;
@@ -513,9 +595,14 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   // NVS_SSD_PP = 1 / 2 / 4 overrides for measurements.
   static const int forced = getenv("NVS_SSD_PP") ? atoi(getenv("NVS_SSD_PP")) : 0;
   int pp = forced ? forced : 2;
-  while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
-  NVS_REQUIRE(ng <= 64 && (int64_t)(P / pp) * ng <= 1024, "%s: state %d x head size %d exceeds one workgroup's registers", who, N, P);
-  const int threads = (P / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
+  if (form == 2) {                                  // (rows need not divide: the kernel guards them; one row more than outputs)
+    while (pp > 1 && ((P + pp - 1) / pp) * ng0 > (pp == 4 ? 320 : 576)) pp >>= 1;
+    if (pp == 1 && P * ng0 > 1024) pp = ((P + 3) / 4) * ng0 <= 320 ? 4 : 1;
+  } else {
+    while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
+  }
+  NVS_REQUIRE(ng <= 64 && (int64_t)((P + pp - 1) / pp) * ng <= 1024, "%s: state %d x head size %d exceeds one workgroup's registers", who, N, P);
+  const int threads = ((P + pp - 1) / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
   int seg_len = 0, nseg = 1;
@@ -526,7 +613,8 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
 #define NVS_SSD_LAUNCH(PPV, MODE, FORM)                                                                                             \
   NVS_DISPATCH(dtype, ssd_scan_kernel<T, PPV, MODE, FORM><<<grid, dim3(threads), lds, (hipStream_t)stream>>>(                        \
                           xbc, (const T*)proj, proj_stride, dt_col, x_col, b_col, c_col, decay, (const T*)dt_bias, (const T*)A_log,   \
-                          (const T*)D, heads, P, N, G, ng, tb, cu_q, ctx0, slot, S, y, seg_len, nseg, ws))
+                          (const T*)D, heads, P, N, G, ng, tb, cu_q, ctx0, slot, S, y, seg_len, nseg, ws, ga.i_col, ga.f_col,                \
+                          (const T*)ga.i_bias, (const T*)ga.f_bias, ga.cap, ga.c_scale, ga.M, ga.den))
 #define NVS_SSD_PASSES(PPV, FORM)   \
   if (seg_len) {                    \
     NVS_SSD_LAUNCH(PPV, 1, FORM);   \
@@ -534,11 +622,13 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   } else {                          \
     NVS_SSD_LAUNCH(PPV, 0, FORM);   \
   }
-#define NVS_SSD_FORMS(PPV)   \
-  if (form == 0) {           \
-    NVS_SSD_PASSES(PPV, 0)   \
-  } else {                   \
-    NVS_SSD_PASSES(PPV, 1)   \
+#define NVS_SSD_FORMS(PPV)        \
+  if (form == 0) {                \
+    NVS_SSD_PASSES(PPV, 0)        \
+  } else if (form == 1) {         \
+    NVS_SSD_PASSES(PPV, 1)        \
+  } else {                        \
+    NVS_SSD_LAUNCH(PPV, 0, 2);    \
   }
   if (pp == 2) {
     NVS_SSD_FORMS(2)
@@ -574,8 +664,25 @@ extern "C" int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_c
                     dv, dk, heads, cu_q, ctx0, slot, nseq, n, max_q, S, y, ws, ws_floats, stream);
 }
 
+extern "C" int nvs_gated_memory_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int64_t i_col,
+                                     int64_t f_col, int dtype, const void* i_bias, const void* f_bias, float cap, float q_scale, int heads,
+                                     int dk, int dv, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
+                                     float* S, float* M, float* y, float* den, void* stream) {
+  NVS_REQUIRE(proj && i_bias && f_bias && cu_q && ctx0 && slot && S && M && y && den, "nvs_gated_memory_scan: null argument");
+  NVS_REQUIRE(cap > 0.f && dv > 0 && dv <= 256, "nvs_gated_memory_scan: cap %g, value size %d", (double)cap, dv);
+  NVS_REQUIRE(v_col >= 0 && k_col >= 0 && q_col >= 0 && i_col >= 0 && f_col >= 0 && v_col + (int64_t)heads * dv <= proj_stride &&
+                  k_col + (int64_t)heads * dk <= proj_stride && q_col + (int64_t)heads * dk <= proj_stride &&
+                  i_col + heads <= proj_stride && f_col + heads <= proj_stride,
+              "nvs_gated_memory_scan: columns beyond the row stride %lld", (long long)proj_stride);
+  GateArgs ga;
+  ga.i_col = i_col, ga.f_col = f_col, ga.i_bias = i_bias, ga.f_bias = f_bias, ga.cap = cap, ga.c_scale = q_scale, ga.M = M, ga.den = den;
+  return ssd_launch(2, "nvs_gated_memory_scan", nullptr, proj, proj_stride, 0, v_col, k_col, q_col, nullptr, dtype, nullptr, nullptr, nullptr,
+                    heads, dv + 1, dk, heads, cu_q, ctx0, slot, nseq, n, 0, S, y, nullptr, 0, stream, ga);
+}
+
 extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,
-                                    float eps, int order, int64_t n, void* out, void* stream) {
+                                    float eps, int order, int64_t n, const float* den, void* out, void* stream) {
+  NVS_REQUIRE(!den || order == 1, "nvs_gated_group_norm: a divisor goes with the order norm, then gate");
   NVS_REQUIRE(y && z && w && out && inner > 0 && groups > 0 && inner % groups == 0 && z_stride >= inner && n >= 0 &&
                   (order == 0 || order == 1),
               "nvs_gated_group_norm: inner %d groups %d order %d", inner, groups, order);
@@ -586,7 +693,8 @@ extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_str
   for (int64_t t0 = 0; t0 < n; t0 += 65535) {
     const int64_t cnt = n - t0 < 65535 ? n - t0 : 65535;
     NVS_DISPATCH(dtype, gated_group_norm_kernel<T><<<dim3(groups, (unsigned)cnt), block, 0, (hipStream_t)stream>>>(
-                            y + t0 * inner, (const T*)z + t0 * z_stride, z_stride, (const T*)w, inner, groups, eps, order, (T*)out + t0 * inner));
+                            y + t0 * inner, (const T*)z + t0 * z_stride, z_stride, (const T*)w, inner, groups, eps, order,
+                            den ? den + t0 * groups : nullptr, (T*)out + t0 * inner));
   }
   return nvs_check_launch("nvs_gated_group_norm");
 }

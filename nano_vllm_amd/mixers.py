@@ -4,6 +4,12 @@
                       query / value head size, optional per-head q/k RMS norm, optional rotation of the leading dimensions
                       in interleaved pairs, optional sigmoid output gate
   AttentionMixer      fused biased q | k | v projection -> WindowAttention -> out projection
+  ConvAttentionMixer  attention whose query and key projections pass a short stateful causal convolution, whose keys (before
+                      rotation) are also its values, with a constant or learned sink in the softmax and a gate per head
+  GatedMemoryCore     matrix memory with exponential input / forget gates held in range by a running maximum (mLSTM style),
+                      per-head RMS norm, sigmoid gate; consumes column ranges of its owner's fused projection
+  AttentionMemoryMixer  position-free attention (query temperature, learned sinks, gated) beside a GatedMemoryCore on the same
+                      input: ONE fused in-projection, two out-projections; the caller adds the two with the design's scales
   LatentAttentionMixer  attention whose keys and values are up-projections of a cached low-rank latent plus one rotated key part
                       shared by the heads; runs in the latent space on WindowAttention's kernels (one kv head), with a query
                       latent, either rotary pairing, optional frequency scaling, window or causal mask, optional per-head
@@ -16,9 +22,11 @@
   ParallelMixer       two mixers on the same input; the caller averages their RMS-normed outputs
   XIELUFeedForward    up -> xIELU -> down
   ClampedGLU          [gate | up] -> min(g, limit) sigmoid(alpha g) (clamp(u) + 1) -> down
+  GeluFeedForward     up -> GELU (tanh form) -> down
   RoutedExperts       mixture of experts (gated SiLU units, or ungated squared-ReLU units): softmax or sigmoid router with a
                       choice-only correction, choice limited to the best groups of experts, weights renormalised or not,
-                      pass-through experts, optional shared expert with a sigmoid gate per token
+                      pass-through experts, optional shared expert with a sigmoid gate per token; or, instead of a router, a
+                      table from token ids to experts with equal weights
 
 Every constant a design may change is a constructor argument. Matrix products are the vendor library's (F.linear /
 baddbmm); everything else is a kernel of libnvl_seq.so (ops_seq). Layers read the step's packed-portion description from
@@ -53,19 +61,29 @@ class WindowAttention(nn.Module):
     """Consumes q | k | v | gate column ranges of the owner's fused projection output."""
 
     def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, window: int, eps: float,
-                 qk_norm: bool = True, block_size: int = 256, chunk: int = 0, rot_dims: int = 0, rot_base: float = 10000.0):
+                 qk_norm: bool = True, block_size: int = 256, chunk: int = 0, rot_dims: int = 0, rot_base: float = 10000.0,
+                 rot_freqs: list | None = None, sink: str | None = None, q_temp: tuple | None = None, gate_per_head: bool = False):
         """window > 0: the last `window` positions are visible; chunk > 0: the positions of the query's own block of `chunk`
         (counted from the start of the sequence); neither: all earlier positions. rot_dims > 0: entries (2i, 2i+1),
-        i < rot_dims / 2, of every query and key head turn by position * rot_base^(-2i / rot_dims)."""
+        i < rot_dims / 2, of every query and key head turn by position * rot_base^(-2i / rot_dims), or by position * rot_freqs[i]
+        when the caller brings its own table of rot_dims / 2 frequencies. sink: "zero" puts one more score of 0 (no value) into every
+        softmax denominator, "learned" a score per head (parameter `sink`, 32-bit). q_temp (coef, every): the query at position p
+        is multiplied by 1 + coef ln(floor((p + 1) / every) + 1). gate_per_head: the gate has one entry per head."""
         super().__init__()
+        assert sink in (None, "zero", "learned") and (rot_freqs is None or len(rot_freqs) == rot_dims // 2)
+        self.gate_per_head, self.q_temp = bool(gate_per_head), (float(q_temp[0]), int(q_temp[1])) if q_temp else None
+        if sink == "learned":
+            self.sink = _param(heads, dtype=torch.float32)
+        else:
+            self.register_buffer("sink", torch.zeros(heads, dtype=torch.float32) if sink else None, persistent=False)
         assert heads % kv_heads == 0 and dim <= 256 and vdim <= 256 and not (window > 0 and chunk > 0)
         assert rot_dims % 2 == 0 and 0 <= rot_dims <= dim
         self.H, self.G, self.d, self.dv = heads, kv_heads, dim, vdim
         self.scale, self.window, self.eps, self.block_size = float(scale), int(window), eps, block_size
         self.chunk = int(chunk)
         # frequencies in double precision on the host, rounded once; angles are position * frequency in 32-bit
-        self.register_buffer("rot_freq", torch.tensor([float(rot_base) ** (-2.0 * i / rot_dims) for i in range(rot_dims // 2)],
-                                                      dtype=torch.float32) if rot_dims else None, persistent=False)
+        freqs = rot_freqs if rot_freqs is not None else [float(rot_base) ** (-2.0 * i / rot_dims) for i in range(rot_dims // 2)]
+        self.register_buffer("rot_freq", torch.tensor(freqs, dtype=torch.float32) if rot_dims else None, persistent=False)
         self.q_norm = _param(dim) if qk_norm else None
         self.k_norm = _param(dim) if qk_norm else None
         self.k_cache = self.v_cache = None            # [pages * block_size, G, d] / [..., G, dv] (values page-transposed), from the runner
@@ -85,7 +103,8 @@ class WindowAttention(nn.Module):
                               self.v_cache, positions, self.rot_freq)
         out = torch.empty(q.shape[0], self.H * self.dv, dtype=q.dtype, device=q.device)
         ops_seq.window_attn(q, self.q_norm, self.eps, gate, self.k_cache, self.v_cache, ctx.block_tables, self.block_size,
-                            ctx.portions, self.H, self.G, self.d, self.dv, self.scale, self.window, out, self.chunk, self.rot_freq)
+                            ctx.portions, self.H, self.G, self.d, self.dv, self.scale, self.window, out, self.chunk, self.rot_freq,
+                            gate_per_head=self.gate_per_head, sink=self.sink, q_temp=self.q_temp)
         return out
 
 
@@ -131,6 +150,139 @@ def rotary_frequencies(dims: int, base: float, scaling: dict | None = None) -> t
     span = max(hi - lo, 0.001)
     ramps = [min(max((i - lo) / span, 0.0), 1.0) for i in range(dims // 2)]
     return [f / factor * r + f * (1.0 - r) for f, r in zip(freq, ramps)], 0.1 * math.log(factor) + 1.0
+
+
+def banded_rotary_frequencies(dims: int, base: float, scaling: dict | None = None) -> list[float]:
+    """Frequencies base^(-2i/dims) of the dims / 2 rotated pairs, in double precision. With `scaling` = {factor, low, high,
+    original} the pairs are treated by wavelength l = 2 pi / f: shorter than original / high they stay, longer than original / low
+    they are divided by `factor`, and between the two marks s = (original / l - low) / (high - low) blends (1 - s) f / factor + s f."""
+    import math
+    freq = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return freq
+    factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    out = []
+    for f in freq:
+        wavelength = 2.0 * math.pi / f
+        if wavelength < original / high:
+            out.append(f)
+        elif wavelength > original / low:
+            out.append(f / factor)
+        else:
+            s_ = (original / wavelength - low) / (high - low)
+            out.append((1.0 - s_) * f / factor + s_ * f)
+    return out
+
+
+class ConvAttentionMixer(nn.Module):
+    """q = conv(W_q h), k = conv(W_k h): a causal convolution of `taps` taps over time on every channel, right after the projection
+    (no bias, no activation; the last taps - 1 projected rows of a sequence are its state). The keys as they leave the convolution
+    are also the values (so vdim == dim and there is no W_v); q and k are then rotated (WindowAttention: rot_dims, rot_freqs).
+    Softmax with a sink (`sink`), head a's output times sigmoid(W_g h)_a, out projection. ONE fused in-projection [q | k | g]."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, taps: int, scale: float, eps: float, block_size: int,
+                 window: int = 0, rot_dims: int = 0, rot_base: float = 10000.0, rot_freqs: list | None = None, sink: str | None = "zero"):
+        super().__init__()
+        assert taps >= 1
+        self.attn = WindowAttention(heads, kv_heads, dim, dim, scale, window, eps, qk_norm=False, block_size=block_size, rot_dims=rot_dims,
+                                    rot_base=rot_base, rot_freqs=rot_freqs, sink=sink, gate_per_head=True)
+        self.q_cols, self.k_cols, self.taps = heads * dim, kv_heads * dim, int(taps)
+        self.channels = self.q_cols + self.k_cols
+        self.in_w = _param(self.channels + heads, width)
+        self.conv_w = _param(self.channels, taps)
+        self.o_w = _param(width, heads * dim)
+        self.conv_state = None
+
+    def state_shapes(self) -> dict:
+        return {"conv_state": (self.taps - 1, self.channels)}
+
+    def named_loaders(self) -> dict:
+        q, c = self.q_cols, self.channels
+        return {"q": _copy_into(self.in_w[:q]), "k": _copy_into(self.in_w[q:c]), "g": _copy_into(self.in_w[c:]),
+                "q.conv": _copy_into(self.conv_w[:q]), "k.conv": _copy_into(self.conv_w[q:]), "o": _copy_into(self.o_w)}
+
+    def forward(self, xh: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        por = get_context().portions
+        q, c = self.q_cols, self.channels
+        proj = F.linear(xh, self.in_w)
+        qk = torch.empty(xh.shape[0], c, dtype=xh.dtype, device=xh.device)
+        ops_seq.causal_conv(proj[:, :c], self.conv_w, None, 0, por, self.conv_state, qk)
+        k = qk[:, q:]
+        return F.linear(self.attn(qk[:, :q], k, k, proj[:, c:], positions), self.o_w)
+
+
+class GatedMemoryCore(nn.Module):
+    """Matrix memory with exponential gates, per head: from the gate pre-activations zi = W_i h + b_i, zf = W_f h + b_f,
+    i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)); a running maximum m' = max(f + m, i) (m = 0 before the first token)
+    keeps exp(f + m - m') and exp(i - m') in range: S <- exp(f + m - m') S + exp(i - m') k v^T, n likewise with k alone,
+    o = S^T q / (max(|n . q|, exp(-m')) + 1e-6) with q = W_q h / sqrt(dim). Every head's o is divided by its root mean square, then
+    times `norm`, times sigmoid(W_g h). State (S with n as one more row, and m) and everything from the gates on are 32-bit.
+    Consumes the columns [v | k | q | g | zi | zf] of its owner's fused projection, starting at col0."""
+
+    def __init__(self, heads: int, dim: int, vdim: int, cap: float, eps: float):
+        super().__init__()
+        self.H, self.d, self.dv, self.cap, self.eps = heads, dim, vdim, float(cap), eps
+        self.cols = (heads * vdim, heads * dim, heads * dim, heads * vdim, heads, heads)          # v | k | q | g | zi | zf
+        self.i_b, self.f_b = _param(heads), _param(heads)
+        self.norm = _param(heads * vdim)
+        self.rec_state = self.max_state = None
+
+    @property
+    def in_width(self) -> int:
+        return sum(self.cols)
+
+    def state_shapes(self) -> dict:
+        return {"rec_state": (self.H, self.dv + 1, self.d), "max_state": (self.H,)}
+
+    def forward(self, proj: torch.Tensor, col0: int) -> torch.Tensor:
+        por = get_context().portions
+        n = proj.shape[0]
+        v, k, q, g, _, _ = self.cols
+        y = torch.empty(n, v, dtype=torch.float32, device=proj.device)
+        den = torch.empty(n, self.H, dtype=torch.float32, device=proj.device)
+        ops_seq.gated_memory_scan(proj, col0, col0 + v, col0 + v + k, col0 + v + k + q + g, col0 + v + k + q + g + self.H, self.i_b,
+                                  self.f_b, self.cap, self.d ** -0.5, self.H, self.d, self.dv, por, self.rec_state, self.max_state, y, den)
+        out = torch.empty(n, v, dtype=proj.dtype, device=proj.device)
+        ops_seq.gated_group_norm(y, proj[:, col0 + v + k + q:col0 + v + k + q + g], self.norm, self.H, self.eps, out, norm_first=True, den=den)
+        return out
+
+
+class AttentionMemoryMixer(nn.Module):
+    """Two mixers on the same input. Left: attention without any rotation, whose queries are multiplied by a temperature that
+    grows with the logarithm of the position (WindowAttention: q_temp), a learned sink per head in the softmax denominator, the
+    concatenated heads times sigmoid(W_g h), out projection. Right: GatedMemoryCore, out projection. ONE fused in-projection
+    [q | k | v | g | right's columns]. Returns both outputs; the caller combines them (each has its own scale)."""
+
+    def __init__(self, width: int, left: dict, right: dict, eps: float, block_size: int):
+        super().__init__()
+        qt = left.get("q_temp")
+        self.attn = WindowAttention(left["heads"], left.get("kv_heads", left["heads"]), left["dim"], left.get("vdim", left["dim"]),
+                                    left["scale"], 0, eps, qk_norm=False, block_size=block_size, sink="learned",
+                                    q_temp=(qt["coef"], qt["every"]) if qt else None)
+        self.mem = GatedMemoryCore(right["heads"], right["dim"], right.get("vdim", right["dim"]), right["gate_cap"], eps)
+        self.cols = list(self.attn.widths) + [self.mem.in_width]
+        self.in_w = _param(sum(self.cols), width)
+        self.left_o = _param(width, self.attn.H * self.attn.dv)
+        self.right_o = _param(width, self.mem.H * self.mem.dv)
+
+    def named_loaders(self) -> dict:
+        q, k, v, g, _ = self.cols
+        o = [0, q, q + k, q + k + v, q + k + v + g]
+        out = {"left.q": _copy_into(self.in_w[o[0]:o[1]]), "left.k": _copy_into(self.in_w[o[1]:o[2]]),
+               "left.v": _copy_into(self.in_w[o[2]:o[3]]), "left.g": _copy_into(self.in_w[o[3]:o[4]]),
+               "left.sink": _copy_into(self.attn.sink), "left.o": _copy_into(self.left_o), "right.o": _copy_into(self.right_o),
+               "right.norm": _copy_into(self.mem.norm), "right.i.b": _copy_into(self.mem.i_b), "right.f.b": _copy_into(self.mem.f_b)}
+        at = o[4]
+        for name, cols in zip(("v", "k", "q", "g", "i", "f"), self.mem.cols):
+            out["right." + name] = _copy_into(self.in_w[at:at + cols])
+            at += cols
+        return out
+
+    def forward(self, xh: torch.Tensor, positions: torch.Tensor | None = None):
+        proj = F.linear(xh, self.in_w)
+        q, k, v, g, _ = self.cols
+        att = self.attn(proj[:, :q], proj[:, q:q + k], proj[:, q + k:q + k + v], proj[:, q + k + v:q + k + v + g])
+        return F.linear(att, self.left_o), F.linear(self.mem(proj, q + k + v + g), self.right_o)
 
 
 class LatentAttentionMixer(nn.Module):
@@ -390,6 +542,23 @@ class XIELUFeedForward(nn.Module):
         return F.linear(ops_seq.xielu(F.linear(xh, self.up), self.act, self.beta), self.down)
 
 
+class GeluFeedForward(nn.Module):
+    """W_down gelu(W_up h), GELU in its tanh form."""
+
+    def __init__(self, width: int, ff: int):
+        super().__init__()
+        self.ff, self.up, self.down = ff, _param(ff, width), _param(width, ff)
+
+    def named_loaders(self) -> dict:
+        return {"up": _copy_into(self.up), "down": _copy_into(self.down)}
+
+    def forward(self, xh: torch.Tensor) -> torch.Tensor:
+        z = F.linear(xh, self.up)
+        act = torch.empty_like(z)
+        ops_seq.glu_act(z, self.ff, act, kind=2)
+        return F.linear(act, self.down)
+
+
 class ClampedGLU(nn.Module):
     """g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit); W_down (g sigmoid(alpha g) (u + 1))."""
 
@@ -417,24 +586,33 @@ class RoutedExperts(nn.Module):
     (`shared_ff`) runs for every token, times sigmoid(w_sg . h). The router's matrix carries w_sg as its last row."""
 
     def __init__(self, width: int, experts: int, ff: int, top: int, scale: float = 1.0, identity: int = 0, group_count: int = 1,
-                 group_keep: int = 1, shared_ff: int = 0, gated: bool = True, sigmoid: bool = False, renorm: bool = True):
+                 group_keep: int = 1, shared_ff: int = 0, gated: bool = True, sigmoid: bool = False, renorm: bool = True,
+                 table_vocab: int = 0, shared_gate: bool = True):
         """gated False: an expert is W_down max(W_up h, 0)^2 (checkpoint names e<i>.up / e<i>.down). sigmoid: scores are each
-        entry's own sigmoid instead of a softmax over the entries. renorm False: the chosen scores are the weights as they are."""
+        entry's own sigmoid instead of a softmax over the entries. renorm False: the chosen scores are the weights as they are.
+        table_vocab > 0: there is no router; row `token id` of `table` [table_vocab, top] (integers) names the token's experts,
+        each with the weight 1 / top, and forward() takes the token ids. shared_gate False: the shared expert is added as it is."""
         super().__init__()
+        self.table_vocab, self.shared_gate = int(table_vocab), bool(shared_gate) and not table_vocab
         self.gated, self.sigmoid, self.renorm = bool(gated), bool(sigmoid), bool(renorm)
         self.E, self.ident, self.ff, self.top, self.scale = experts, identity, ff, top, float(scale)
         self.count, self.keep, self.shared_ff = group_count, group_keep, shared_ff
         total = experts + identity
         assert total % group_count == 0 and 1 <= group_keep <= group_count and top <= group_keep * (total // group_count)
-        self.router = _param(total + (1 if shared_ff else 0), width, dtype=torch.float32)
-        self.correction = _param(total, dtype=torch.float32)
+        if table_vocab:
+            assert identity == 0 and group_count == 1
+            self.table = _param(table_vocab, top, dtype=torch.int32)
+        else:
+            self.router = _param(total + (1 if shared_ff and self.shared_gate else 0), width, dtype=torch.float32)
+            self.correction = _param(total, dtype=torch.float32)
         self.w_gu, self.w_down = _param(experts, (2 if gated else 1) * ff, width), _param(experts, width, ff)
         if shared_ff:
             self.s_gu, self.s_down = _param(2 * shared_ff, width), _param(width, shared_ff)
 
     def named_loaders(self) -> dict:
         total, ff = self.E + self.ident, self.ff
-        out = {"router": _copy_into(self.router[:total]), "correction": _copy_into(self.correction)}
+        out = {"table": _copy_into(self.table)} if self.table_vocab else \
+            {"router": _copy_into(self.router[:total]), "correction": _copy_into(self.correction)}
         for e in range(self.E):
             if self.gated:
                 out[f"e{e}.gate"] = _copy_into(self.w_gu[e, :ff])
@@ -445,14 +623,20 @@ class RoutedExperts(nn.Module):
         if self.shared_ff:
             sf = self.shared_ff
             out.update({"shared.gate": _copy_into(self.s_gu[:sf]), "shared.up": _copy_into(self.s_gu[sf:]),
-                        "shared.down": _copy_into(self.s_down), "shared.sg": _copy_into(self.router[total:])})
+                        "shared.down": _copy_into(self.s_down)})
+            if self.shared_gate:
+                out["shared.sg"] = _copy_into(self.router[total:])
         return out
 
-    def forward(self, xh: torch.Tensor) -> torch.Tensor:
+    def forward(self, xh: torch.Tensor, tokens: torch.Tensor | None = None) -> torch.Tensor:
         n, width = xh.shape
         total = self.E + self.ident
-        z = F.linear(xh.float(), self.router)                                     # 32-bit, [n, total (+ 1: the shared gate)]
-        ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale, self.sigmoid, self.renorm)
+        if self.table_vocab:
+            z = None
+            ids, wts = ops_seq.moe_table_route(tokens, self.table, 1.0 / self.top)
+        else:
+            z = F.linear(xh.float(), self.router)                                 # 32-bit, [n, total (+ 1: the shared gate)]
+            ids, wts = ops_seq.moe_route(z, total, self.correction, self.top, self.count, self.keep, self.scale, self.sigmoid, self.renorm)
         per_expert = n * self.top // self.E                 # rows an expert gets on average: the tile height follows it
         plan = ops_seq.moe_plan(ids, self.E, 128 if per_expert >= 256 else (64 if per_expert >= 64 else 16))
         act = torch.empty(plan.cap, self.ff, dtype=xh.dtype, device=xh.device)
@@ -463,7 +647,7 @@ class RoutedExperts(nn.Module):
         if self.shared_ff:
             sact = torch.empty(n, self.shared_ff, dtype=xh.dtype, device=xh.device)
             ops_seq.glu_act(F.linear(xh, self.s_gu), self.shared_ff, sact, kind=0)
-            shared, gate = F.linear(sact, self.s_down), z[:, total:]
+            shared, gate = F.linear(sact, self.s_down), (z[:, total:] if self.shared_gate else None)
         out = torch.empty(n, width, dtype=xh.dtype, device=xh.device)
         ops_seq.moe_combine(rows, plan, wts, xh, shared, gate, out)
         return out

@@ -15,7 +15,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 
 SIGNATURES = {
@@ -25,17 +25,20 @@ SIGNATURES = {
     "nvs_norm_residual": (c_int, [_P, _P, _P, _P, _P, _I, _L, _I, _F, _P, _P, _P]),
     "nvs_scalar_norm_rows": (c_int, [_P, _P, _L, _I, _P, _I, _F, _P, _P]),
     "nvs_xielu": (c_int, [_P, _P, _F, _I, _L, _P, _P]),
-    "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _P]),
+    "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _I, _P]),
+    "nvs_sandwich_norm": (c_int, [_P, _P, _F, _P, _F, _P, _P, _L, _P, _F, _I, _I, _F, _P, _P]),
+    "nvs_gated_memory_scan": (c_int, [_P, _L, _L, _L, _L, _L, _L, _I, _P, _P, _F, _F, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P, _P, _P]),
+    "nvs_moe_table_route": (c_int, [_P, _P, _L, _I, _F, _P, _P, _P]),
     "nvs_rglru_scan_workspace": (c_int64, [_I, _I, _L]),
     "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_ssd_scan_workspace": (c_int64, [_I, _I, _I, _I, _L]),
     "nvs_ssd_scan": (c_int, [_P, _P, _L, _L, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
     "nvs_decay_scan": (c_int, [_P, _L, _L, _L, _L, _I, _P, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
-    "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _I, _L, _P, _P]),
+    "nvs_gated_group_norm": (c_int, [_P, _P, _L, _I, _P, _I, _I, _F, _I, _L, _P, _P, _P]),
     "nvs_knorm_kvstore": (c_int, [_P, _P, _L, _I, _P, _F, _I, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P]),
     "nvs_window_attn_force_scalar": (None, [_I]),
     "nvs_window_attn": (c_int, [_P, _L, _P, _F, _P, _L, _I, _I, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _I, _I, _I, _I, _F, _I,
-                                _I, _P, _I, _P, _P]),
+                                _I, _P, _I, _P, _F, _I, _P, _P]),
     "nvs_add_group_norm": (c_int, [_P, _P, _F, _P, _P, _L, _P, _I, _I, _I, _F, _I, _P, _P]),
     "nvs_scale_softcap": (c_int, [_P, _I, _F, _F, _L, _P, _P]),
     "nvs_latent_prep": (c_int, [_P, _L, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _F, _F, _I, _P, _P, _P, _L, _P]),
@@ -163,14 +166,15 @@ def xielu(z: torch.Tensor, pq: torch.Tensor, beta: float = 0.5) -> torch.Tensor:
 
 def causal_conv(inp: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, act: int, por: Portions, state: torch.Tensor,
                 out: torch.Tensor):
-    """inp: [n, channels] view (unit column stride) of a projection output; state [nslots, taps - 1, channels] fp32."""
+    """inp: [n, channels] view (unit column stride) of a projection output; state [nslots, taps - 1, channels] fp32; out 32-bit or
+    of inp's type."""
     lib = load_library()
     channels, taps = w.shape
     assert inp.shape == (por.n, channels) and inp.stride(1) == 1 and w.is_contiguous()
     assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (taps - 1, channels)
-    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (por.n, channels)
+    assert out.dtype in (torch.float32, inp.dtype) and out.is_contiguous() and out.shape == (por.n, channels)
     _check(lib.nvs_causal_conv(_ptr(inp), inp.stride(0), _same(inp, w, b), _ptr(w), _ptr(b), channels, taps, act, _ptr(por.cu_q),
-                               _ptr(por.ctx0), _ptr(por.slot), _ptr(por.tseq), por.nseq, por.n, _ptr(state), _ptr(out), _stream()))
+                               _ptr(por.ctx0), _ptr(por.slot), _ptr(por.tseq), por.nseq, por.n, _ptr(state), _ptr(out), _code(out), _stream()))
 
 
 def rglru_scan(gates: torch.Tensor, u: torch.Tensor, ypre: torch.Tensor, lam: torch.Tensor, c: float, blocks: int, por: Portions,
@@ -207,14 +211,16 @@ def ssd_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias, A_log,
 
 
 def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
-                     norm_first: bool = False):
-    """out = group_rms(y * silu(z)) * w, or with norm_first group_rms(y) * w * sigmoid(z)."""
+                     norm_first: bool = False, den: torch.Tensor | None = None):
+    """out = group_rms(y * silu(z)) * w, or with norm_first group_rms(y) * w * sigmoid(z); den [n, groups] (32-bit, norm_first only):
+    group g of row t is divided by den[t, g] before anything else."""
     lib = load_library()
     n, inner = y.shape
     assert y.dtype == torch.float32 and y.is_contiguous() and z.shape == (n, inner) and z.stride(1) == 1
     assert w.numel() == inner and out.shape == (n, inner) and out.is_contiguous()
+    assert den is None or (norm_first and den.dtype == torch.float32 and den.shape == (n, groups) and den.is_contiguous())
     _check(lib.nvs_gated_group_norm(_ptr(y), _ptr(z), z.stride(0), _same(z, w, out), _ptr(w), inner, groups, eps, int(norm_first), n,
-                                    _ptr(out), _stream()))
+                                    _ptr(den), _ptr(out), _stream()))
 
 
 def _rotation(rot_freq: torch.Tensor | None) -> int:
@@ -244,20 +250,25 @@ def knorm_kvstore(k: torch.Tensor, v: torch.Tensor, knorm: torch.Tensor | None, 
 
 def window_attn(q: torch.Tensor, qnorm: torch.Tensor | None, eps: float, gate: torch.Tensor | None, k_cache, v_cache,
                 block_tables: torch.Tensor, block_size: int, por: Portions, H: int, G: int, d: int, dv: int, scale: float,
-                window: int, out: torch.Tensor, chunk: int = 0, rot_freq: torch.Tensor | None = None, gate_per_head: bool = False):
+                window: int, out: torch.Tensor, chunk: int = 0, rot_freq: torch.Tensor | None = None, gate_per_head: bool = False,
+                sink: torch.Tensor | None = None, q_temp: tuple[float, int] | None = None):
     """window > 0: the last `window` positions; chunk > 0: the query's own block of `chunk` positions; neither: causal.
     rot_freq [r / 2] (32-bit): the first r entries of every query head turn in interleaved pairs by position * rot_freq.
-    gate [n, H * dv], or [n, H] with gate_per_head: out *= sigmoid(gate)."""
+    gate [n, H * dv], or [n, H] with gate_per_head: out *= sigmoid(gate). sink [H] (32-bit): head h's softmax denominator also holds
+    exp(sink[h]). q_temp (coef, every): the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)."""
     lib = load_library()
     n = por.n
     assert q.shape == (n, H * d) and q.stride(1) == 1 and out.shape == (n, H * dv) and out.is_contiguous()
     assert gate is None or (gate.shape == (n, H if gate_per_head else H * dv) and gate.stride(1) == 1)
     assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and block_tables.shape[0] >= por.nseq
     assert tuple(k_cache.shape[1:]) == (G, d) and tuple(v_cache.shape[1:]) == (G, dv)
+    assert sink is None or (sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous() and sink.is_cuda)
+    qt_coef, qt_every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 0)
     _check(lib.nvs_window_attn(_ptr(q), q.stride(0), _ptr(qnorm), eps, _ptr(gate), gate.stride(0) if gate is not None else 0,
                                int(gate_per_head), _same(q, qnorm, gate, k_cache, v_cache, out), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                block_tables.stride(0), block_size, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.tseq), por.nseq, n, H,
-                               G, d, dv, scale, window, chunk, _ptr(rot_freq), _rotation(rot_freq), _ptr(out), _stream()))
+                               G, d, dv, scale, window, chunk, _ptr(rot_freq), _rotation(rot_freq), _ptr(sink), qt_coef, qt_every, _ptr(out),
+                               _stream()))
 
 
 def add_group_norm(x: torch.Tensor, w: torch.Tensor | None, groups: int, eps: float, out: torch.Tensor | None,
@@ -285,6 +296,50 @@ def group_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, w: t
     assert rows is not None or nrows <= x.shape[0]
     _check(lib.nvs_add_group_norm(_ptr(x), None, 1.0, None, _ptr(rows), nrows, _ptr(w), _same(out, w), x.shape[1], groups, eps, int(center),
                                   _ptr(out), _stream()))
+
+
+def sandwich_norm(x: torch.Tensor, a: torch.Tensor | None, wa: torch.Tensor | None, w: torch.Tensor | None, eps: float,
+                  out: torch.Tensor | None, a2: torch.Tensor | None = None, a_mult: float = 1.0, a2_mult: float = 1.0, w_off: float = 1.0):
+    """x += rms(a_mult * a + a2_mult * a2) * (w_off + wa) (in place; a None: no add), then out = rms(x) * (w_off + w) (out None: no
+    second norm)."""
+    lib = load_library()
+    n, width = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert a is None or (a.shape == x.shape and a.is_contiguous() and wa is not None and wa.numel() == width)
+    assert a2 is None or (a is not None and a2.shape == x.shape and a2.is_contiguous())
+    assert out is None or (out.shape == x.shape and out.is_contiguous() and w is not None and w.numel() == width)
+    ref = out if out is not None else a
+    assert ref is not None, "nothing to do"
+    _check(lib.nvs_sandwich_norm(_ptr(x), _ptr(a), a_mult, _ptr(a2), a2_mult, _ptr(wa) if a is not None else None, None, n,
+                                 _ptr(w) if out is not None else None, w_off, _same(ref, a, a2, wa if a is not None else None,
+                                                                                   w if out is not None else None, out), width, eps, _ptr(out), _stream()))
+
+
+def offset_norm_rows(x: torch.Tensor, rows: torch.Tensor | None, nrows: int, w: torch.Tensor, eps: float, out: torch.Tensor, w_off: float = 1.0):
+    """out[r] = rms(x[rows[r]]) * (w_off + w) (rows None: row r)."""
+    lib = load_library()
+    assert x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == (nrows, x.shape[1])
+    assert rows is None or (rows.dtype == torch.int32 and rows.numel() >= nrows)
+    assert rows is not None or nrows <= x.shape[0]
+    _check(lib.nvs_sandwich_norm(_ptr(x), None, 1.0, None, 1.0, None, _ptr(rows), nrows, _ptr(w), w_off, _same(out, w), x.shape[1], eps,
+                                 _ptr(out), _stream()))
+
+
+def gated_memory_scan(proj: torch.Tensor, v_col: int, k_col: int, q_col: int, i_col: int, f_col: int, i_bias: torch.Tensor,
+                      f_bias: torch.Tensor, cap: float, q_scale: float, heads: int, dk: int, dv: int, por: Portions, S: torch.Tensor,
+                      M: torch.Tensor, y: torch.Tensor, den: torch.Tensor):
+    """The matrix memory with exponential gates (see include/nvl_seq.h): S [nslots, heads, dv + 1, dk] and M [nslots, heads] are the
+    state; y [n, heads * dv] receives the numerators, den [n, heads] the divisors."""
+    lib = load_library()
+    n = por.n
+    assert proj.shape[0] == n and proj.stride(1) == 1 and i_bias.numel() == heads and f_bias.numel() == heads
+    assert S.dtype == torch.float32 and S.is_contiguous() and tuple(S.shape[1:]) == (heads, dv + 1, dk)
+    assert M.dtype == torch.float32 and M.is_contiguous() and tuple(M.shape[1:]) == (heads,) and M.shape[0] == S.shape[0]
+    assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, heads * dv)
+    assert den.dtype == torch.float32 and den.is_contiguous() and den.shape == (n, heads)
+    _check(lib.nvs_gated_memory_scan(_ptr(proj), proj.stride(0), v_col, k_col, q_col, i_col, f_col, _same(proj, i_bias, f_bias), _ptr(i_bias),
+                                     _ptr(f_bias), cap, q_scale, heads, dk, dv, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n,
+                                     _ptr(S), _ptr(M), _ptr(y), _ptr(den), _stream()))
 
 
 def scale_softcap(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
@@ -355,10 +410,11 @@ def decay_scan(proj: torch.Tensor, v_col: int, k_col: int, q_col: int, decay: to
 
 
 def glu_act(gu: torch.Tensor, ff: int, out: torch.Tensor, kind: int = 0, limit: float = 0.0, alpha: float = 1.0):
-    """gu [n, 2 ff] = [gate | up] -> out [n, ff]. kind 0: silu(g) u; kind 1: min(g, limit) sigmoid(alpha g) (clamp(u) + 1)."""
+    """gu [n, 2 ff] = [gate | up] -> out [n, ff]. kind 0: silu(g) u; kind 1: min(g, limit) sigmoid(alpha g) (clamp(u) + 1);
+    kind 2: gu [n, ff], no gate: the tanh form of GELU."""
     lib = load_library()
     n = gu.shape[0]
-    assert gu.shape[1] == 2 * ff and gu.stride(1) == 1 and out.shape == (n, ff) and out.is_contiguous()
+    assert gu.shape[1] == (1 if kind == 2 else 2) * ff and gu.stride(1) == 1 and out.shape == (n, ff) and out.is_contiguous()
     _check(lib.nvs_glu_act(_ptr(gu), gu.stride(0), _same(gu, out), ff, kind, limit, alpha, n, _ptr(out), _stream()))
 
 
@@ -374,6 +430,17 @@ def moe_route(z: torch.Tensor, total: int, correction: torch.Tensor | None, top:
     wts = torch.empty(n, top, dtype=torch.float32, device=z.device)
     _check(lib.nvs_moe_route(_ptr(z), z.stride(0), _ptr(correction), n, total, top, count, keep, scale, int(sigmoid), int(renorm), _ptr(ids),
                              _ptr(wts), _stream()))
+    return ids, wts
+
+
+def moe_table_route(tokens: torch.Tensor, table: torch.Tensor, weight: float):
+    """tokens [n] int64, table [vocab, top] int32 -> (ids [n, top] = table[tokens], weights [n, top] = weight)."""
+    lib = load_library()
+    n, top = tokens.numel(), table.shape[1]
+    assert tokens.dtype == torch.int64 and tokens.is_contiguous() and table.dtype == torch.int32 and table.is_contiguous()
+    ids = torch.empty(n, top, dtype=torch.int32, device=tokens.device)
+    wts = torch.empty(n, top, dtype=torch.float32, device=tokens.device)
+    _check(lib.nvs_moe_table_route(_ptr(tokens), _ptr(table), n, top, weight, _ptr(ids), _ptr(wts), _stream()))
     return ids, wts
 
 
@@ -415,8 +482,8 @@ def moe_combine(rows: torch.Tensor, plan: MoePlan, wts: torch.Tensor, h: torch.T
     top = wts.shape[1]
     assert rows.stride(1) == 1 and rows.shape[1] == width and h.stride(1) == 1 and out.shape == (n, width) and out.is_contiguous()
     assert wts.dtype == torch.float32 and wts.is_contiguous() and plan.pair_row.shape == (n, top)
-    assert shared is None or (shared.shape == (n, width) and shared.is_contiguous() and shared_gate.dtype == torch.float32
-                              and shared_gate.shape[0] == n)
+    assert shared is None or (shared.shape == (n, width) and shared.is_contiguous())
+    assert shared_gate is None or (shared is not None and shared_gate.dtype == torch.float32 and shared_gate.shape[0] == n)
     _check(lib.nvs_moe_combine(_ptr(rows), rows.stride(0), _ptr(plan.pair_row), _ptr(wts), top, _ptr(h), h.stride(0), _ptr(shared),
                                _ptr(shared_gate), shared_gate.stride(0) if shared_gate is not None else 0, _same(rows, h, shared, out), n,
                                width, _ptr(out), _stream()))

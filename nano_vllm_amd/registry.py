@@ -68,6 +68,16 @@ def _pefazen_build(config, dtype=None):
     return PefazenForCausalLM(config, dtype)
 
 
+def _lobidra_config(path: str, raw: dict):
+    from .lobidra import LobidraConfig
+    return LobidraConfig(raw)
+
+
+def _lobidra_build(config, dtype=None):
+    from .lobidra import LobidraForCausalLM
+    return LobidraForCausalLM(config, dtype)
+
+
 REGISTRY: dict[str, ModelSpec] = {
     "Qwen3ForCausalLM": ModelSpec("Qwen3ForCausalLM", _qwen3_config, _qwen3_build),
     "Qwen2ForCausalLM": ModelSpec("Qwen2ForCausalLM", _qwen3_config, _qwen3_build),      # same module tree, biased qkv, no q/k norm
@@ -76,6 +86,8 @@ REGISTRY: dict[str, ModelSpec] = {
     "Nokipel": ModelSpec("Nokipel", _nokipel_config, _nokipel_build, stateful=True, block_multiple=16,
                          dtypes=("bfloat16", "float32")),
     "Pefazen": ModelSpec("Pefazen", _pefazen_config, _pefazen_build, stateful=True, block_multiple=16,
+                         dtypes=("bfloat16", "float32")),
+    "Lobidra": ModelSpec("Lobidra", _lobidra_config, _lobidra_build, stateful=True, block_multiple=16,
                          dtypes=("bfloat16", "float32")),
 }
 
