@@ -18,8 +18,11 @@ __device__ __forceinline__ int vis_lo(int p, int window, int chunk) {
 
 // factor on the query at position p: 1 + coef * ln(floor((p + 1) / every) + 1) — a temperature that grows with the logarithm of the
 // position, in steps of `every` positions (every == 0: none)
+// (positions are below 2^24, so p + 1 and `every` are exact in 32-bit floats and the correctly rounded quotient has the integer
+// quotient's floor: a float division instead of the long expansion of an integer one)
 __device__ __forceinline__ float query_temp(int p, float coef, int every) {
-  return every > 0 ? 1.f + coef * logf((float)((p + 1) / every) + 1.f) : 1.f;
+  if (every <= 0) return 1.f;
+  return 1.f + coef * logf(floorf((float)(p + 1) / (float)every) + 1.f);
 }
 
 // one wavefront per (token, kv head)
@@ -260,12 +263,13 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(
   const int lo = vis_lo(p_first, window, chunk);
   const int lo_hi = vis_lo(c0 + tile * QW + QW - 1, window, chunk);      // the tile's last query sees the least far back
   const int32_t* bt = block_tables + (int64_t)s * bt_stride;
+  const float sink_m = sink ? sink[h] : -1e30f, sink_l = sink && gq == 0 ? 1.f : 0.f;      // (see the LDS form below)
   float m[QT], lsum[QT];
   f32x4_t oacc[QT][DVB];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    m[t] = sink ? sink[h] : -1e30f;                 // a sink: a score in the denominator without a value (counted once: by gq 0)
-    lsum[t] = sink && gq == 0 ? 1.f : 0.f;
+    m[t] = sink_m;
+    lsum[t] = sink_l;
 #pragma unroll
     for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -473,12 +477,15 @@ __global__ __launch_bounds__(256) void window_attn_mfma_lds_kernel(
         qb[t][c][e + 1] = (bf16_t)b;
       }
   }
+  // a sink: a score in the denominator without a value; the running maximum and sum start from it (the sum once per query: in
+  // the lanes with gq 0). All tiles of a wavefront belong to one head, except in the packed form, which has one tile.
+  const float sink_m = sink ? sink[hq[0]] : -1e30f, sink_l = sink && gq == 0 ? 1.f : 0.f;
   float m[QT], lsum[QT];
   f32x4_t oacc[QT][DVB];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    m[t] = sink ? sink[hq[t]] : -1e30f;             // a sink: a score in the denominator without a value (counted once: by gq 0)
-    lsum[t] = sink && gq == 0 ? 1.f : 0.f;
+    m[t] = sink_m;
+    lsum[t] = sink_l;
 #pragma unroll
     for (int db = 0; db < DVB; ++db) oacc[t][db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }

@@ -348,3 +348,64 @@ def test_attention_in_the_latent_space_is_the_same_sum_reordered():
             p = np.exp(sc - sc.max())
             got[t, a] = w["uv"].reshape(H, dv, r)[a] @ ((p / p.sum()) @ lat[keys]) / (1.0 + np.exp(-(h[t] @ w["g"][a])))
     assert np.abs(got.reshape(n, H * dv) - want).max() < 1e-12
+
+
+# ---- Lobidra --------------------------------------------------------------------------------------------------------------
+def lbd_raw():
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": 20},
+           "mixer": {"heads": 4, "kv_heads": 2, "dim": 6, "vdim": 6, "conv": 3, "scale": 0.4,
+                     "rot": {"dims": 4, "base": 100.0, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 16}}}}
+    par = {"type": "parallel", "mlp": {"kind": "moe", "expert": {"ff": 10}, "router": {"experts": 3, "top": 2}, "shared": {"ff": 12}},
+           "mixer": {"left": {"heads": 2, "kv_heads": 1, "dim": 4, "vdim": 8, "scale": 0.5, "q_temp": {"coef": 0.25, "every": 8}},
+                     "right": {"heads": 3, "dim": 4, "vdim": 2, "gate_cap": 9.0}, "left_scale": 0.5, "right_scale": 2.0}}
+    return {"architecture": "Lobidra", "layers": [att, par, dict(att, weights_of=0), dict(par, weights_of=1, mlp=par["mlp"])],
+            "norm": {"eps": 1e-5}, "vocab": 29, "width": 16, "embedding": {"scale": 4.0}}
+
+
+def test_lobidra_registry_and_config_checks(tmp_path):
+    from nano_vllm_amd.registry import REGISTRY, resolve
+    (tmp_path / "config.json").write_text(json.dumps(lbd_raw()))
+    spec, cfg = resolve(str(tmp_path))
+    assert spec is REGISTRY["Lobidra"] and spec.stateful and set(spec.dtypes) == {"bfloat16", "float32"}
+    assert (cfg.vocab_size, cfg.hidden_size, cfg.embedding_scale, cfg.eps) == (29, 16, 4.0, 1e-5)
+    assert [cfg.owner(i) for i in range(4)] == [0, 1, 0, 1]
+    cases = [(lambda r: r["layers"][0].update(type="lstm"), "mixer type"), (lambda r: r["layers"][0].update(mlp={"kind": "glu"}), "feed-forward kind"),
+             (lambda r: r["layers"][2].update(weights_of=3), "weights_of"), (lambda r: r["layers"][3].update(weights_of=2), "weights_of"),
+             (lambda r: r["layers"][2].update(weights_of=1), "another type"), (lambda r: r["layers"][0]["mixer"].update(vdim=8), "vdim")]
+    for change, msg in cases:
+        raw = json.loads(json.dumps(lbd_raw()))
+        change(raw)
+        (tmp_path / "config.json").write_text(json.dumps(raw))
+        with pytest.raises(ValueError, match=msg):
+            resolve(str(tmp_path))
+
+
+def test_lobidra_checkpoint_names_loaders_and_weights_shared_between_layers():
+    """Every tensor the synthetic checkpoint writes has a loader in the model and the other way round; a layer that runs with another
+    layer's weights has no tensors and holds the very same parameter objects."""
+    from nano_vllm_amd.lobidra import LobidraConfig, LobidraForCausalLM, random_tensors, tensor_shapes
+    raw = lbd_raw()
+    model = LobidraForCausalLM(LobidraConfig(raw), torch.float32, block_size=16)
+    loaders, shapes = model.named_loaders(), tensor_shapes(raw)
+    assert set(loaders) == set(shapes) and not any(n.startswith(("l2.", "l3.")) for n in shapes)
+    assert "l0.mix.v" not in shapes and "l0.mix.q.conv" in shapes and "l1.mlp.router" not in shapes and shapes["l1.mlp.table"] == (29, 2)
+    tensors = random_tensors(raw, seed=3)
+    with torch.no_grad():
+        for name, t in tensors.items():
+            assert tuple(t.shape) == tuple(shapes[name]) and t.dtype == (torch.int32 if name.endswith(".table") else torch.bfloat16)
+            loaders[name](t)
+    assert all(len(set(row)) == 2 and max(row) < 3 for row in tensors["l1.mlp.table"].tolist())
+    a, p, a2, p2 = model.layers
+    assert a2.mixer.in_w is a.mixer.in_w and a2.norm1b is a.norm1b and p2.mlp.w_gu is p.mlp.w_gu and p2.mixer.attn.sink is p.mixer.attn.sink
+    assert sum(p_.numel() for p_ in set(model.parameters())) == sum(int(torch.tensor(s).prod()) for s in shapes.values())
+    # fused in-projections: [q | k | gate per head] and [q | k | v | g || v | k | q | g | zi | zf]
+    assert a.mixer.in_w.shape == (24 + 12 + 4, 16) and a.mixer.conv_w.shape == (36, 3) and a.mixer.state_shapes() == {"conv_state": (2, 36)}
+    assert torch.equal(a.mixer.in_w[24:36], tensors["l0.mix.k"].float()) and torch.equal(a.mixer.conv_w[24:], tensors["l0.mix.k.conv"].float())
+    assert a.mixer.attn.kv_shapes() == ((2, 6), (2, 6)) and a.mixer.attn.sink.tolist() == [0.0] * 4 and a.mixer.attn.gate_per_head
+    assert p.mixer.in_w.shape == (8 + 4 + 8 + 16 + 6 + 12 + 12 + 6 + 3 + 3, 16) and p.mixer.attn.q_temp == (0.25, 8)
+    assert torch.equal(p.mixer.in_w[36 + 6 + 12:36 + 6 + 24], tensors["l1.mix.right.q"].float())
+    assert torch.equal(p.mixer.in_w[-3:], tensors["l1.mix.right.f"].float()) and torch.equal(p.mixer.attn.sink, tensors["l1.mix.left.sink"].float())
+    assert p.mixer.mem.state_shapes() == {"rec_state": (3, 3, 4), "max_state": (3,)} and p.scales == (0.5, 2.0) and a.scales == (1.0, 1.0)
+    assert p.mlp.table_vocab == 29 and not p.mlp.shared_gate and not hasattr(p.mlp, "router") and a.mlp.up.shape == (20, 16)
+    # the rotation's table: wavelengths 2 pi and 20 pi against marks at 8 and 16 positions: the first pair stays, the second is slowed
+    assert a.mixer.attn.rot_freq.tolist() == [1.0, pytest.approx(0.05)]
