@@ -29,8 +29,8 @@ driver's fields it carries
                  race keys with the draws replayed (a by-product of the cpu_baseline leg: the timed
                  oracle pass is teacher-forced with the engine's tokens).
 
-`python bench.py --compare-families [--families pefazen,nokipel,foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a
-line of its own (metric "family_compare"): prefill and decode throughput of the Pefazen, Nokipel and Foduzen families at layer
+`python bench.py --compare-families [--families lobidra,pefazen,nokipel,foduzen,qwen3] [--sizes 1k,4k]` is a different measurement with a
+line of its own (metric "family_compare"): prefill and decode throughput of the Lobidra, Pefazen, Nokipel and Foduzen families at layer
 sizes of real models beside Qwen3 at equal width and depth. The default command above is unchanged by it.
 """
 from __future__ import annotations
@@ -89,9 +89,9 @@ def parse():
     ap.add_argument("--kv-cache-dtype", default="bf16", choices=["bf16", "fp8"],
                     help="fp8: opt-in OCP e4m3 KV cache (outside the reference's numerics; never the headline)")
     ap.add_argument("--compare-families", action="store_true",
-                    help="instead of the headline workload: prefill and decode throughput of the Pefazen, Nokipel and Foduzen families at "
+                    help="instead of the headline workload: prefill and decode throughput of the Lobidra, Pefazen, Nokipel and Foduzen families at "
                          "layer sizes of real models (random weights) beside Qwen3 models of equal width / depth, one JSON line")
-    ap.add_argument("--families", default="pefazen,nokipel,foduzen,qwen3", help="with --compare-families: which of the four to run")
+    ap.add_argument("--families", default="lobidra,pefazen,nokipel,foduzen,qwen3", help="with --compare-families: which of the five to run")
     ap.add_argument("--sizes", default="1k,4k", help="with --compare-families: layer sizes to run (1k, 4k)")
     return ap.parse_args()
 
@@ -148,6 +148,29 @@ def pefazen_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, 
             "logit_scale": 1.0, "logit_softcap": 30.0}
 
 
+def lobidra_config(width: int, ff: int, heads: int, kv_heads: int, layers: int, vocab: int) -> dict:
+    """Layers of a real model's size: attention layers with 128-wide heads, a convolution of 4 taps on queries and keys, half of
+    every head rotated with scaled frequencies and 32 table-chosen experts of a quarter of the dense width (4 per token) plus a
+    shared one; parallel layers with 128-wide attention heads (temperature every 1,024 positions) beside 128 x 128 memory heads
+    (as many as make the model's width) and a dense feed-forward. The two kinds alternate; from the third layer on a layer runs
+    with the weights of the layer two before it."""
+    att = {"type": "attention",
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+                     "rot": {"dims": 64, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}},
+           "mlp": {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}}}
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "q_temp": {"coef": 0.1, "every": 1024}},
+                     "right": {"heads": width // 128, "dim": 128, "vdim": 128, "gate_cap": 15.0}, "left_scale": 0.7, "right_scale": 0.7}}
+    out = []
+    for i in range(layers):
+        layer = dict(att if i % 2 == 0 else par)
+        if i >= 2:
+            layer["weights_of"] = i % 2
+        out.append(layer)
+    return {"architecture": "Lobidra", "embedding": {"scale": 1.0}, "layers": out, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+
+
 FAMILY_SIZES = {   # name: (width, ff, heads, kv heads, layers, the Qwen3 shape of the same width / depth)
     "1k": (1024, 3072, 16, 8, 4, "qwen3-0.6b-4l"),
     "4k": (4096, 12288, 32, 8, 2, "qwen3-8b-2l"),
@@ -169,8 +192,9 @@ def compare_families(args) -> dict:
         width, ff, heads, kv, layers, qname = FAMILY_SIZES[size]
         for family in args.families.split(","):
             path = os.path.join(tempfile.gettempdir(), f"nvl_cmp_{family}_{size}")
-            if family in ("foduzen", "nokipel", "pefazen"):
-                raw = {"foduzen": foduzen_config, "nokipel": nokipel_config, "pefazen": pefazen_config}[family](width, ff, heads, kv, layers, vocab)
+            if family in ("foduzen", "nokipel", "pefazen", "lobidra"):
+                raw = {"foduzen": foduzen_config, "nokipel": nokipel_config, "pefazen": pefazen_config,
+                       "lobidra": lobidra_config}[family](width, ff, heads, kv, layers, vocab)
                 os.makedirs(path, exist_ok=True)
                 with open(os.path.join(path, "config.json"), "w") as fh:
                     json.dump(raw, fh)

@@ -168,8 +168,9 @@ constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken togethe
 // FORM 2: the matrix memory with exponential gates. Per head and token, from the gate pre-activations zi, zf (columns i_col / f_col
 // + head of the projection output, plus a bias each): i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)); with a running
 // maximum m (0 at a sequence's start) m' = max(f + m, i), S <- exp(f + m - m') S + exp(i - m') k v^T, n likewise with k alone. The
-// walk is the same with x = v, B = k, C = q * c_scale, decay exp(f + m - m'), step exp(i - m') — ONE thread turns the round's gates
-// into these, token after token, while the others stage the operands — and n is simply one more row of the state, whose "value" is
+// walk is the same with x = v, B = k, C = q * c_scale, decay exp(f + m - m'), step exp(i - m') — per round of tokens the gates are
+// computed a token per thread, ONE thread walks the maximum through them, and the exponentials are again a token per thread —
+// and n is simply one more row of the state, whose "value" is
 // the constant 1: the kernel sees P = dv + 1 rows (state memory [heads][dv + 1][dk], M [nslots][heads] holds m). It writes the
 // numerators S^T q to y [n, heads * dv] and den [n, heads] = max(|n . q|, exp(-m')) + 1e-6; the division is left to the norm that
 // follows. Never segmented (a segment's maximum depends on all tokens before it).
@@ -200,7 +201,8 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
   if (mode == 1 && last && seg > 0) return;         // nobody starts from the last segment's state
   float* wst = ws + ((int64_t)(s * heads + h) * (nseg + 1)) * P * N + (int64_t)p * N + g * SSD_R;   // entry e: + e P N
   float* wdec = ws + (int64_t)gridDim.y * heads * (nseg + 1) * P * N + (int64_t)(s * heads + h) * (nseg + 1);
-  const int NP = NG * SSD_R, P4 = (P + 3) & ~3, per = P4 + 2 * NP + 4;    // every part starts 16-byte aligned
+  // every part starts 16-byte aligned; the x part also covers the rows of the last thread that lie beyond P (zeros: form 2's row count need not divide)
+  const int NP = NG * SSD_R, P4 = ((P + PP - 1) / PP * PP + 3) & ~3, per = P4 + 2 * NP + 4;
   const int inner = heads * P, grp = h / (heads / G);
   const int64_t row = inner + 2 * G * N;
   float A = 0.f, Dh = 0.f, dtb = 0.f, fixed_decay = 1.f;
@@ -301,33 +303,7 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
         kind = 3;
       }
       float v[SSD_TB];
-      if (FORM == 2 && kind == 2) {
-        // this thread alone: the round's gates -> step, decay and exp(-m) of every token, in order (m runs through the portion)
-        float zi[SSD_TB], zf[SSD_TB];
-#pragma unroll
-        for (int k = 0; k < SSD_TB; ++k) {
-          zi[k] = zf[k] = 0.f;
-          if (k < cnt) {
-            zi[k] = ldf(proj + (tb + k) * proj_stride + i_col + h);
-            zf[k] = ldf(proj + (tb + k) * proj_stride + f_col + h);
-          }
-        }
-#pragma unroll
-        for (int k = 0; k < SSD_TB; ++k) {
-          if (k < cnt) {
-            const float gi = cap * tanhf((zi[k] + bi) / cap);
-            const float zc = cap * tanhf((zf[k] + bf) / cap);
-            const float gf = fminf(zc, 0.f) - log1pf(expf(-fabsf(zc)));          // log sigmoid
-            const float mn = fmaxf(gf + mrun, gi);
-            lds[k * per + c] = expf(gi - mn);
-            lds[k * per + c + 1] = expf(gf + mrun - mn);
-            lds[k * per + c + 2] = expf(-mn);
-            mrun = mn;
-          }
-        }
-        continue;
-      }
-      if (FORM == 2 && c > P4 + 2 * NP) continue;   // (decay, exp(-m) and the spare entry belong to the thread beside)
+      if (FORM == 2 && c >= P4 + 2 * NP) continue;  // (step, decay, exp(-m): from the gates, below)
 #pragma unroll
       for (int k = 0; k < SSD_TB; ++k) {
         v[k] = 0.f;
@@ -361,7 +337,34 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
         }
       }
     }
+    float* gates = lds + P4 + 2 * NP;               // FORM 2: per token (+ k * per) the gates i, f -> step, decay, exp(-m)
+    if (FORM == 2) {
+      for (int k = tid; k < cnt; k += nthreads) {   // the gates themselves, a token per thread
+        const float zi = ldf(proj + (tb + k) * proj_stride + i_col + h), zf = ldf(proj + (tb + k) * proj_stride + f_col + h);
+        const float zc = cap * tanhf((zf + bf) / cap);
+        gates[k * per] = cap * tanhf((zi + bi) / cap);
+        gates[k * per + 1] = fminf(zc, 0.f) - log1pf(expf(-fabsf(zc)));          // log sigmoid
+      }
+    }
     __syncthreads();
+    if (FORM == 2) {
+      if (tid == 0) {                               // the running maximum, token after token: an add and a max each
+        for (int k = 0; k < cnt; ++k) {
+          const float mn = fmaxf(gates[k * per + 1] + mrun, gates[k * per]);
+          gates[k * per + 2] = mrun;
+          gates[k * per + 3] = mn;
+          mrun = mn;
+        }
+      }
+      __syncthreads();
+      for (int k = tid; k < cnt; k += nthreads) {
+        const float gi = gates[k * per], gf = gates[k * per + 1], mb = gates[k * per + 2], mn = gates[k * per + 3];
+        gates[k * per] = expf(gi - mn);
+        gates[k * per + 1] = expf(gf + mb - mn);
+        gates[k * per + 2] = expf(-mn);
+      }
+      __syncthreads();
+    }
     // one token: S <- dA S + dt B x; returns this thread's share of y = S . C for each of its rows
     auto token = [&](int k, float (&part)[PP], float (&xs)[PP]) {
       const float* tp = lds + k * per;
@@ -374,7 +377,7 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
       for (int r = 0; r < SSD_R; ++r) bv[r] = Bp[r], cv[r] = Cp[r];
 #pragma unroll
       for (int i = 0; i < PP; ++i) {
-        const float xv = (FORM != 2 || p + i < P) ? tp[p + i] : 0.f;
+        const float xv = tp[p + i];
         const float dx = dt * xv;
         float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
@@ -447,7 +450,7 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
 #pragma unroll
     for (int i = 0; i < PP; ++i)
       if (FORM != 2 || p + i < P) store16(Sh + (int64_t)i * N, st[i]);
-    if (FORM == 2 && tid == (P4 + 2 * NP) % nthreads) M[(int64_t)slot[s] * heads + h] = mrun;      // the thread that kept it
+    if (FORM == 2 && tid == 0) M[(int64_t)slot[s] * heads + h] = mrun;      // the thread that kept it
   }
 }
 
@@ -602,7 +605,7 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
     while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
   }
   NVS_REQUIRE(ng <= 64 && (int64_t)((P + pp - 1) / pp) * ng <= 1024, "%s: state %d x head size %d exceeds one workgroup's registers", who, N, P);
-  const int threads = ((P + pp - 1) / pp) * ng, per = ((P + 3) & ~3) + 2 * ng * SSD_R + 4;
+  const int threads = ((P + pp - 1) / pp) * ng, per = (((P + pp - 1) / pp * pp + 3) & ~3) + 2 * ng * SSD_R + 4;
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
   int seg_len = 0, nseg = 1;

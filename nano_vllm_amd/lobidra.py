@@ -252,8 +252,8 @@ def random_tensors(raw: dict, seed: int = 0) -> dict[str, torch.Tensor]:
         if leaf == "table":
             layer = raw["layers"][int(name.split(".")[0][1:])]
             experts = layer["mlp"]["router"]["experts"]
-            rows = [torch.randperm(experts, generator=gen)[:shape[1]] for _ in range(shape[0])]
-            out[name] = torch.stack(rows).to(torch.int32)
+            order = torch.rand(shape[0], experts, generator=gen, dtype=torch.float32, device="cpu").argsort(dim=1)
+            out[name] = order[:, :shape[1]].to(torch.int32)             # a row: the first `top` of a random order of the experts
             continue
         r = torch.randn(shape, generator=gen, dtype=torch.float32, device="cpu")
         if name.endswith("right.norm"):
