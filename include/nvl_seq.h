@@ -117,11 +117,14 @@ int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t
  * q (times q_scale), k (dk per head) and v (dv per head) being columns q_col / k_col / v_col (+ head * size) of proj, read as they
  * are. y [n, heads * dv] receives the numerators S^T q, den [n, heads] the divisors max(|n . q|, exp(-m')) + 1e-6 (both 32-bit; the
  * norm that follows divides: nvs_gated_group_norm's `den`). State: S [nslots, heads, dv + 1, dk] (row dv is n; dk fastest) and
- * M [nslots, heads], advanced. The walk is nvs_ssd_scan's, one workgroup per (portion, head); never segmented. dv <= 256. */
+ * M [nslots, heads], advanced. The walk is nvs_ssd_scan's, one workgroup per (portion, head), and so are the segments for long
+ * portions (`ws`: nvs_gated_memory_scan_workspace floats; NULL: never; a segment's local state is combined with what came before
+ * it through its own maximum and the sum of its log forget gates). dv <= 256. */
+int64_t nvs_gated_memory_scan_workspace(int heads, int dk, int dv, int nseq, int64_t max_q);
 int nvs_gated_memory_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int64_t i_col, int64_t f_col,
                           int dtype, const void* i_bias, const void* f_bias, float cap, float q_scale, int heads, int dk, int dv,
-                          const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n, float* S, float* M, float* y,
-                          float* den, void* stream);
+                          const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n, int64_t max_q, float* S,
+                          float* M, float* y, float* den, float* ws, int64_t ws_floats, void* stream);
 
 /* order 0: out = group_rms(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row by its own root mean
  * square. order 1: out = group_rms(y) * w * sigmoid(z): the norm first. y [n, inner] 32-bit; z [n, inner] with row stride z_stride

@@ -6,7 +6,7 @@
 
 namespace {
 
-constexpr int MAX_TAPS = 8;
+constexpr int MAX_TAPS = 16;
 
 // ---- causal convolution -------------------------------------------------------------------------------------------
 // one thread per (token, channel); inputs before the portion come from the slot's tail (or are zero at a sequence start)
@@ -173,9 +173,12 @@ constexpr int SSD_SB = 8;      // tokens whose cross-lane sums are taken togethe
 // and n is simply one more row of the state, whose "value" is
 // the constant 1: the kernel sees P = dv + 1 rows (state memory [heads][dv + 1][dk], M [nslots][heads] holds m). It writes the
 // numerators S^T q to y [n, heads * dv] and den [n, heads] = max(|n . q|, exp(-m')) + 1e-6; the division is left to the norm that
-// follows. Never segmented (a segment's maximum depends on all tokens before it).
+// follows. Segments: a segment scanned from nothing (its own maximum starting at "minus infinity") ends with a local state L, a
+// local maximum ml and the sum F of its log forget gates; behind a state (S, m) the true state after it is m' = max(m + F, ml),
+// S' = exp(m + F - m') S + exp(ml - m') L — the same sum of terms, scaled by another maximum — so mode 2 combines the segments
+// before its own in order and then walks its tokens as usual (`ws` holds F and ml beside every local state).
 template <typename T, int PP, int MODE, int FORM = 0>     // PP head-size entries per thread: the B / C values read from LDS serve PP state rows
-__global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)) : (PP == 4 ? 256 : (PP == 2 ? 512 : 1024))) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
+__global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 512 : (PP == 2 ? 576 : 1024)) : (PP == 4 ? 256 : (PP == 2 ? 512 : 1024))) void ssd_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ proj, int64_t proj_stride, int64_t dt_col,
                                 int64_t x_col, int64_t b_col, int64_t c_col, const float* __restrict__ decay,
                                 const T* __restrict__ dt_bias, const T* __restrict__ A_log, const T* __restrict__ Dp, int heads,
                                 int P, int N, int G, int NG, int TB, const int32_t* __restrict__ cu_q,
@@ -200,7 +203,8 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
   const bool last = q1 == p1;
   if (mode == 1 && last && seg > 0) return;         // nobody starts from the last segment's state
   float* wst = ws + ((int64_t)(s * heads + h) * (nseg + 1)) * P * N + (int64_t)p * N + g * SSD_R;   // entry e: + e P N
-  float* wdec = ws + (int64_t)gridDim.y * heads * (nseg + 1) * P * N + (int64_t)(s * heads + h) * (nseg + 1);
+  constexpr int WD = FORM == 2 ? 3 : 1;             // numbers kept beside a segment's state: its decay product, or F and ml
+  float* wdec = ws + (int64_t)gridDim.y * heads * (nseg + 1) * P * N + (int64_t)(s * heads + h) * (nseg + 1) * WD;
   // every part starts 16-byte aligned; the x part also covers the rows of the last thread that lie beyond P (zeros: form 2's row count need not divide)
   const int NP = NG * SSD_R, P4 = ((P + PP - 1) / PP * PP + 3) & ~3, per = P4 + 2 * NP + 4;
   const int inner = heads * P, grp = h / (heads / G);
@@ -216,10 +220,15 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
   const bool fresh = ctx0[s] == 0;
   // FORM 2: the running maximum (kept by the one thread that turns gates into decays), the gates' biases, rows beyond P are idle
   const int Py = FORM == 2 ? P - 1 : P;             // rows that are outputs
-  float mrun = 0.f, bi = 0.f, bf = 0.f;
+  float mrun = 0.f, bi = 0.f, bf = 0.f, fsum = 0.f;
   if (FORM == 2) {
     bi = ldf(i_bias + h), bf = ldf(f_bias + h);
     if (!fresh) mrun = M[(int64_t)slot[s] * heads + h];
+    if (mode == 1) {                                // the portion's starting maximum for mode 2; a segment by itself starts from none
+      if (seg == 0 && tid == 0) wdec[1] = mrun;
+      mrun = -1e30f;
+    }
+    if (mode == 2) mrun = wdec[1];
   }
   const bool vec = (N & 3) == 0;                    // a thread's 16 entries are then four aligned 16-byte pieces
   auto load16 = [&](const float* src, float (&dst)[SSD_R]) {
@@ -250,20 +259,31 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
   for (int i = 0; i < PP; ++i) {
 #pragma unroll
     for (int r = 0; r < SSD_R; ++r) st[i][r] = 0.f;
+    const bool row_ok = FORM != 2 || p + i < P;     // (form 2's last thread may hold rows beyond the state)
     if (mode == 2) {
-      load16(wst + (int64_t)i * N, st[i]);          // S_0, then the segments before this one
+      if (row_ok) load16(wst + (int64_t)i * N, st[i]);          // S_0, then the segments before this one
+      float mk = FORM == 2 ? wdec[1] : 0.f;
       for (int k = 0; k < seg; ++k) {
         float lk[SSD_R];
-        load16(wst + (int64_t)(k + 1) * P * N + (int64_t)i * N, lk);
-        const float dk = wdec[k + 1];
 #pragma unroll
-        for (int r = 0; r < SSD_R; ++r) st[i][r] = dk * st[i][r] + lk[r];
+        for (int r = 0; r < SSD_R; ++r) lk[r] = 0.f;
+        if (row_ok) load16(wst + (int64_t)(k + 1) * P * N + (int64_t)i * N, lk);
+        float dk = wdec[(k + 1) * WD], bk = 1.f;
+        if (FORM == 2) {
+          const float F = wdec[(k + 1) * WD], ml = wdec[(k + 1) * WD + 1];
+          const float mn = fmaxf(mk + F, ml);
+          dk = expf(mk + F - mn), bk = expf(ml - mn);
+          mk = mn;
+        }
+#pragma unroll
+        for (int r = 0; r < SSD_R; ++r) st[i][r] = dk * st[i][r] + bk * lk[r];
       }
+      if (FORM == 2) mrun = mk;
     } else if (!fresh && (mode == 0 || seg == 0) && (FORM != 2 || p + i < P)) {
       load16(Sh + (int64_t)i * N, st[i]);
     }
     if (mode == 1 && seg == 0) {                    // the portion's starting state, for mode 2
-      store16(wst + (int64_t)i * N, st[i]);
+      if (row_ok) store16(wst + (int64_t)i * N, st[i]);
 #pragma unroll
       for (int r = 0; r < SSD_R; ++r) st[i][r] = 0.f;
     }
@@ -353,6 +373,7 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
           const float mn = fmaxf(gates[k * per + 1] + mrun, gates[k * per]);
           gates[k * per + 2] = mrun;
           gates[k * per + 3] = mn;
+          fsum += gates[k * per + 1];
           mrun = mn;
         }
       }
@@ -444,8 +465,12 @@ __global__ __launch_bounds__(FORM == 2 ? (PP == 4 ? 320 : (PP == 2 ? 576 : 1024)
   }
   if (mode == 1) {
 #pragma unroll
-    for (int i = 0; i < PP; ++i) store16(wst + (int64_t)(seg + 1) * P * N + (int64_t)i * N, st[i]);
-    if (tid == 0) wdec[seg + 1] = dprod;
+    for (int i = 0; i < PP; ++i)
+      if (FORM != 2 || p + i < P) store16(wst + (int64_t)(seg + 1) * P * N + (int64_t)i * N, st[i]);
+    if (tid == 0) {
+      if (FORM == 2) wdec[(seg + 1) * WD] = fsum, wdec[(seg + 1) * WD + 1] = mrun;
+      else wdec[seg + 1] = dprod;
+    }
   } else if (last) {
 #pragma unroll
     for (int i = 0; i < PP; ++i)
@@ -573,6 +598,12 @@ extern "C" int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int
   return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)P * N + 1) : 0;
 }
 
+extern "C" int64_t nvs_gated_memory_scan_workspace(int heads, int dk, int dv, int nseq, int64_t max_q) {
+  int seg_len, nseg;
+  ssd_plan(heads, nseq, max_q, &seg_len, &nseg);
+  return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)(dv + 1) * dk + 3) : 0;
+}
+
 // what only the matrix memory (form 2) passes
 struct GateArgs {
   int64_t i_col = 0, f_col = 0;
@@ -599,8 +630,7 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   static const int forced = getenv("NVS_SSD_PP") ? atoi(getenv("NVS_SSD_PP")) : 0;
   int pp = forced ? forced : 2;
   if (form == 2) {                                  // (rows need not divide: the kernel guards them; one row more than outputs)
-    while (pp > 1 && ((P + pp - 1) / pp) * ng0 > (pp == 4 ? 320 : 576)) pp >>= 1;
-    if (pp == 1 && P * ng0 > 1024) pp = ((P + 3) / 4) * ng0 <= 320 ? 4 : 1;
+    if (((P + 1) / 2) * ng0 > 576) pp = ((P + 3) / 4) * ng0 <= 512 ? 4 : 1;
   } else {
     while (pp > 1 && (P % pp != 0 || (P / pp) * ng0 > (pp == 4 ? 256 : 512))) pp >>= 1;
   }
@@ -610,7 +640,8 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   const size_t lds = (size_t)tb * per * sizeof(float);
   int seg_len = 0, nseg = 1;
   if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
-  NVS_REQUIRE(!seg_len || ws_floats >= nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n),
+  NVS_REQUIRE(!seg_len || ws_floats >= (form == 2 ? nvs_gated_memory_scan_workspace(heads, N, P - 1, nseq, max_q > 0 ? max_q : n)
+                                                   : nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n)),
               "%s: workspace of %lld floats is too small", who, (long long)ws_floats);
   const dim3 grid(heads, (unsigned)nseq, seg_len ? nseg : 1);
 #define NVS_SSD_LAUNCH(PPV, MODE, FORM)                                                                                             \
@@ -631,7 +662,7 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   } else if (form == 1) {         \
     NVS_SSD_PASSES(PPV, 1)        \
   } else {                        \
-    NVS_SSD_LAUNCH(PPV, 0, 2);    \
+    NVS_SSD_PASSES(PPV, 2)        \
   }
   if (pp == 2) {
     NVS_SSD_FORMS(2)
@@ -670,7 +701,7 @@ extern "C" int nvs_decay_scan(const void* proj, int64_t proj_stride, int64_t v_c
 extern "C" int nvs_gated_memory_scan(const void* proj, int64_t proj_stride, int64_t v_col, int64_t k_col, int64_t q_col, int64_t i_col,
                                      int64_t f_col, int dtype, const void* i_bias, const void* f_bias, float cap, float q_scale, int heads,
                                      int dk, int dv, const int32_t* cu_q, const int32_t* ctx0, const int32_t* slot, int nseq, int64_t n,
-                                     float* S, float* M, float* y, float* den, void* stream) {
+                                     int64_t max_q, float* S, float* M, float* y, float* den, float* ws, int64_t ws_floats, void* stream) {
   NVS_REQUIRE(proj && i_bias && f_bias && cu_q && ctx0 && slot && S && M && y && den, "nvs_gated_memory_scan: null argument");
   NVS_REQUIRE(cap > 0.f && dv > 0 && dv <= 256, "nvs_gated_memory_scan: cap %g, value size %d", (double)cap, dv);
   NVS_REQUIRE(v_col >= 0 && k_col >= 0 && q_col >= 0 && i_col >= 0 && f_col >= 0 && v_col + (int64_t)heads * dv <= proj_stride &&
@@ -680,7 +711,7 @@ extern "C" int nvs_gated_memory_scan(const void* proj, int64_t proj_stride, int6
   GateArgs ga;
   ga.i_col = i_col, ga.f_col = f_col, ga.i_bias = i_bias, ga.f_bias = f_bias, ga.cap = cap, ga.c_scale = q_scale, ga.M = M, ga.den = den;
   return ssd_launch(2, "nvs_gated_memory_scan", nullptr, proj, proj_stride, 0, v_col, k_col, q_col, nullptr, dtype, nullptr, nullptr, nullptr,
-                    heads, dv + 1, dk, heads, cu_q, ctx0, slot, nseq, n, 0, S, y, nullptr, 0, stream, ga);
+                    heads, dv + 1, dk, heads, cu_q, ctx0, slot, nseq, n, max_q, S, y, ws, ws_floats, stream, ga);
 }
 
 extern "C" int nvs_gated_group_norm(const float* y, const void* z, int64_t z_stride, int dtype, const void* w, int inner, int groups,

@@ -27,7 +27,9 @@ SIGNATURES = {
     "nvs_xielu": (c_int, [_P, _P, _F, _I, _L, _P, _P]),
     "nvs_causal_conv": (c_int, [_P, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _L, _P, _P, _I, _P]),
     "nvs_sandwich_norm": (c_int, [_P, _P, _F, _P, _F, _P, _P, _L, _P, _F, _I, _I, _F, _P, _P]),
-    "nvs_gated_memory_scan": (c_int, [_P, _L, _L, _L, _L, _L, _L, _I, _P, _P, _F, _F, _I, _I, _I, _P, _P, _P, _I, _L, _P, _P, _P, _P, _P]),
+    "nvs_gated_memory_scan_workspace": (c_int64, [_I, _I, _I, _I, _L]),
+    "nvs_gated_memory_scan": (c_int, [_P, _L, _L, _L, _L, _L, _L, _I, _P, _P, _F, _F, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _P, _P,
+                                      _L, _P]),
     "nvs_moe_table_route": (c_int, [_P, _P, _L, _I, _F, _P, _P, _P]),
     "nvs_rglru_scan_workspace": (c_int64, [_I, _I, _L]),
     "nvs_rglru_scan": (c_int, [_P, _P, _P, _L, _I, _P, _F, _I, _I, _P, _P, _P, _I, _L, _L, _P, _P, _P, _L, _P]),
@@ -337,9 +339,11 @@ def gated_memory_scan(proj: torch.Tensor, v_col: int, k_col: int, q_col: int, i_
     assert M.dtype == torch.float32 and M.is_contiguous() and tuple(M.shape[1:]) == (heads,) and M.shape[0] == S.shape[0]
     assert y.dtype == torch.float32 and y.is_contiguous() and y.shape == (n, heads * dv)
     assert den.dtype == torch.float32 and den.is_contiguous() and den.shape == (n, heads)
+    need = 0 if torch.cuda.is_current_stream_capturing() else lib.nvs_gated_memory_scan_workspace(heads, dk, dv, por.nseq, por.max_q)
+    ws = torch.empty(need, dtype=torch.float32, device=proj.device) if need else None
     _check(lib.nvs_gated_memory_scan(_ptr(proj), proj.stride(0), v_col, k_col, q_col, i_col, f_col, _same(proj, i_bias, f_bias), _ptr(i_bias),
                                      _ptr(f_bias), cap, q_scale, heads, dk, dv, _ptr(por.cu_q), _ptr(por.ctx0), _ptr(por.slot), por.nseq, n,
-                                     _ptr(S), _ptr(M), _ptr(y), _ptr(den), _stream()))
+                                     por.max_q, _ptr(S), _ptr(M), _ptr(y), _ptr(den), _ptr(ws), need, _stream()))
 
 
 def scale_softcap(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:

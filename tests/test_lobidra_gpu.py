@@ -509,6 +509,27 @@ def test_unequal_requests_in_one_batch_equal_each_alone_with_pages_and_slots_reu
         llm.exit()
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+def test_a_long_portion_scanned_in_segments_beside_a_short_one(checkpoints, variant):
+    """600 tokens in one step: the matrix memory cuts such a portion into segments that are scanned twice; the request beside it
+    has one segment. The decoded tokens after it continue from the state the segmented pass left."""
+    path = checkpoints[variant]
+    ref = plain.Model.load(path)
+    g = torch.Generator().manual_seed(21)
+    long, short = (torch.randint(0, ref.cfg["vocab"], (n,), generator=g).tolist() for n in (604, 9))
+    wl, ws = ref.run(long), ref.run(short)
+    scale = float(wl.std())
+    llm = engine(path, "float32", pages=42)
+    try:
+        out = llm.replay_step([{"id": "l", "tokens": long[:600], "want": [0, 300, 511, 512, 599]}, {"id": "s", "tokens": short[:5], "want": [4]}])
+        assert rel(out[:5], wl[[0, 300, 511, 512, 599]], scale) <= 5e-5 and rel(out[5:], ws[[4]], scale) <= 5e-5
+        for i in range(4):
+            out = llm.replay_step([{"id": "s", "tokens": [short[5 + i]], "want": [0]}, {"id": "l", "tokens": [long[600 + i]], "want": [0]}])
+            assert rel(out[:1], ws[[5 + i]], scale) <= 5e-5 and rel(out[1:], wl[[600 + i]], scale) <= 5e-5, i
+    finally:
+        llm.exit()
+
+
 def test_long_decoding_across_many_pages(checkpoints):
     path = checkpoints[2]
     ref = plain.Model.load(path)
