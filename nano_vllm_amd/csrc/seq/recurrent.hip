@@ -575,13 +575,15 @@ extern "C" int nvs_rglru_scan(const float* gates, const float* u, const void* yp
 }
 
 // Segments for long portions when (portion, head) pairs alone would leave compute units idle: seg_len 0 = none.
-static void ssd_plan(int heads, int nseq, int64_t max_q, int* seg_len, int* nseg) {
+static void ssd_plan(int heads, int nseq, int64_t max_q, int* seg_len, int* nseg, int full_at = 512) {
   *seg_len = 0;
   *nseg = 1;
   const int64_t pairs = (int64_t)heads * nseq;
   // (measured, 8 x 2048 tokens: 128 pairs 11.8 ms per step unsegmented -> 9.8 with 1,024 workgroups -> 9.3 with 2,048; 512 pairs,
   //  two workgroups per CU already, LOSE with two or four segments each: 18.7 -> 19.8 - 20.0)
-  if (pairs >= 512 || max_q < 512) return;
+  // (the matrix memory's workgroups are larger — one per compute unit — and 256 pairs already lose: 8 x 2048 tokens x 32 heads of
+  //  128 x 128 take 3.9 ms in one pass, 2.0 + 3.9 ms in segments; 64 pairs 3.85 ms against 0.45 + 0.95; it passes full_at = 192)
+  if (pairs >= full_at || max_q < 512) return;
   const int target = (int)((2048 + pairs - 1) / pairs);     // segments wanted per portion
   int64_t sl = (max_q + target - 1) / target;
   sl = (sl + 15) / 16 * 16;
@@ -600,7 +602,7 @@ extern "C" int64_t nvs_ssd_scan_workspace(int heads, int P, int N, int nseq, int
 
 extern "C" int64_t nvs_gated_memory_scan_workspace(int heads, int dk, int dv, int nseq, int64_t max_q) {
   int seg_len, nseg;
-  ssd_plan(heads, nseq, max_q, &seg_len, &nseg);
+  ssd_plan(heads, nseq, max_q, &seg_len, &nseg, 192);
   return seg_len ? (int64_t)nseq * heads * (nseg + 1) * ((int64_t)(dv + 1) * dk + 3) : 0;
 }
 
@@ -639,7 +641,7 @@ static int ssd_launch(int form, const char* who, const float* xbc, const void* p
   const int tb = SSD_TB;                            // tokens per LDS round
   const size_t lds = (size_t)tb * per * sizeof(float);
   int seg_len = 0, nseg = 1;
-  if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg);
+  if (ws) ssd_plan(heads, nseq, max_q > 0 ? max_q : n, &seg_len, &nseg, form == 2 ? 192 : 512);
   NVS_REQUIRE(!seg_len || ws_floats >= (form == 2 ? nvs_gated_memory_scan_workspace(heads, N, P - 1, nseq, max_q > 0 ? max_q : n)
                                                    : nvs_ssd_scan_workspace(heads, P, N, nseq, max_q > 0 ? max_q : n)),
               "%s: workspace of %lld floats is too small", who, (long long)ws_floats);
